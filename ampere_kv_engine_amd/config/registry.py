@@ -13,6 +13,7 @@ import os
 from typing import Protocol
 
 from .keranex import KeranexConfig
+from .lirulix import LirulixConfig
 from .qwen3 import ConfigError, Qwen3Config
 from .tukevik import TukevikConfig
 from .specs import ModelSpec
@@ -65,3 +66,4 @@ def load_config(folder: str) -> ArchitectureConfig:
 register_architecture(Qwen3Config.architecture, Qwen3Config)
 register_architecture(KeranexConfig.architecture, KeranexConfig)
 register_architecture(TukevikConfig.architecture, TukevikConfig)
+register_architecture(LirulixConfig.architecture, LirulixConfig)

@@ -49,10 +49,15 @@ class LayerSpec:
 class RunEntry:
     """One entry of the run order.  `layer` indexes `ModelSpec.layers` (a layer may be named twice);
     `cache_layer` names the layer whose cache the mixer uses (its own by default); `writes_cache` is False
-    for an entry that only reads what another entry wrote."""
+    for an entry that only reads what another entry wrote.  A layer that runs several times with the same weights
+    and a cache or state of its own each time names the time in `cache_copy` (0, 1, ...): every (cache_layer,
+    cache_copy) is a cache of its own.  `adds_row`: before this entry runs, row `adds_row` of the model's table of
+    vectors (`ModelSpec.pass_vectors`) is added to every token's residual sum."""
     layer: int
     cache_layer: int
     writes_cache: bool = True
+    cache_copy: int = 0
+    adds_row: int | None = None
 
 
 @dataclass(frozen=True)
@@ -67,11 +72,20 @@ class ModelSpec:
     head: PartSpec
     eos_token_ids: tuple[int, ...] = ()
     max_position: int | None = None
+    pass_vectors: PartSpec | None = None        # a table [rows, hidden] of vectors that run-order entries add (`adds_row`)
 
     def __post_init__(self):
         for entry in self.run_order:
             if not (0 <= entry.layer < len(self.layers) and 0 <= entry.cache_layer < len(self.layers)):
                 raise ValueError(f"run order entry {entry} names a layer outside 0..{len(self.layers) - 1}")
+            if entry.cache_copy < 0:
+                raise ValueError(f"run order entry {entry} names a negative copy of its cache")
+            if entry.adds_row is not None and (self.pass_vectors is None or not 0 <= entry.adds_row < self.pass_vectors["rows"]):
+                raise ValueError(f"run order entry {entry} adds a row that the model's table of vectors does not have")
+
+    def cache_key(self, entry: RunEntry) -> int:
+        """The number under which the cache manager keeps the cache that `entry` uses."""
+        return entry.cache_layer + entry.cache_copy * len(self.layers)
 
 
 def default_run_order(num_layers: int) -> tuple[RunEntry, ...]:

@@ -18,11 +18,24 @@ int akv_embed_pairs(const int* ids, const void* table, const void* pairs, int dt
 int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots, int* slot_words, int seqs,
                         hipStream_t stream);
 // stream [tokens, hidden] float32.  With `delta` (dtype): stream += delta / rms(delta) * post_weight (or += delta where
-// post_weight is null: stream += delta_scale * delta).  With `out` (dtype): out = stream / rms(stream) * pre_weight,
-// rounded once.
+// post_weight is null: stream += delta_scale * delta).  With `offset` [hidden]: stream += offset, every row, after the
+// branch.  With `out` (dtype): out = stream / rms(stream) * pre_weight, rounded once.
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      float delta_scale, hipStream_t stream);
+                      float delta_scale, const float* offset, hipStream_t stream);
+// out[n] = table[id] / rms(table[id]) * weight: the start of a residual sum that is normed before the first layer (an id
+// of -1: the token chosen last for the row's request, where the slot words are given)
+int akv_embed_normed(const int* ids, const void* table, int dtype, const float* weight, float eps, float* out, int tokens,
+                     int hidden, int vocab, const int* seq_of_token, const int* seq_slots, const int* slot_words,
+                     hipStream_t stream);
+// out [tokens, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:]; activation 0: silu, 1: the tanh form of gelu
+int akv_gated_activation(const void* gate_up, void* out, int dtype, long tokens, int inter, int activation,
+                         hipStream_t stream);
+// maps [tokens, heads, 2, vdim] -> out [tokens, heads, vdim] = (a1 - lambda[0] a2) / rms(.) * after *
+// sigmoid(gates[t * gate_stride + gate_at + h * vdim + i])
+int akv_difference_norm_gate(const void* maps, const float* lambda, float eps, float after, const void* gates,
+                             long gate_stride, long gate_at, void* out, int dtype, long tokens, int heads, int vdim,
+                             hipStream_t stream);
 
 // out = a * scale_a + b * scale_b (float32 arithmetic, one rounding)
 int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, void* out, int dtype, long count,
@@ -33,20 +46,27 @@ int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, v
 // by their root mean square per head (where `normed`) go to q_out [tokens, q_heads, dim]; with `slot_map` the keys, the
 // same way, and the values go to the token's slot of the pages: keys [pages, kv_heads, page, dim], values [pages,
 // kv_heads, vdim, page].
+// `maps` > 1: a head's queries and keys are `maps` vectors of `dim` side by side (rows [q (q_heads x maps x dim) | k (kv_heads
+// x maps x dim) | v]), each normed and rotated for itself; key pages [pages, kv_heads, page, maps x dim].  `table`
+// [table_positions, rot_dims / 2, 2] (cos, sin; null: no rotation): a vector's first rot_dims dimensions are rotated by the
+// token's position, dimension i with i + rot_dims / 2.
 int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
                         int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
-                        long num_pages, void* q_out, hipStream_t stream);
+                        long num_pages, void* q_out, int maps, const float* table, int table_positions, int rot_dims,
+                        const int* positions, hipStream_t stream);
 // out [tokens, q_heads, vdim].  score = (q . k) * scale, then softcap * tanh(score / softcap) where softcap > 0; a query at
 // position p sees the keys j <= p with j > p - window (window > 0) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
 // with `sink` the softmax's denominator has one more term exp(0); with `gates` head h's output is multiplied by
 // sigmoid(gates[t * gate_stride + gate_at + h]).  A token's outputs lie at out + t * out_stride, times out_scale.
-// `row_waves` (1 .. 16) waves share a token's head: each takes every row_waves-th tile of 64 keys.
+// `row_waves` (1 .. 16) waves share a token's head: each takes every row_waves-th tile of 64 keys.  `sink_logits` [q_heads]
+// float32 (with `sink`): the extra term is exp(sink_logits[h]).  `maps` > 1: `q_heads` counts query vectors, `maps` a head
+// (out [tokens, q_heads, vdim] accordingly); vector v reads vector v % maps of its key head's record and the head's values.
 int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
                              int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
                              int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
-                             hipStream_t stream);
+                             const float* sink_logits, int maps, hipStream_t stream);
 
 // The same for rows first_row .. tokens - 1 of a bfloat16 step, on the matrix cores: keys and values 32, 64, 128 or 256
 // wide, pages of a multiple of 16 tokens (-2 otherwise); a request's rows follow each other in the order of their positions.
@@ -55,7 +75,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
                               float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
-                              hipStream_t stream);
+                              const float* sink_logits, int maps, hipStream_t stream);
 
 // ---- mixers with a state of fixed size (recurrent_mixers.hip) ----------------------------------------------------------
 // projected [tokens, stride]: rows [q | k (heads x dim each) | v | g (heads x vdim each)].  q and k are rotated over their
@@ -82,6 +102,20 @@ int akv_retention_chunked(const void* projected, long stride, int dtype, int seq
 int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const float* gate_bias, const float* rate,
                           const void* y, long y_stride, int seqs, int channels, int blocks, int runs, float* state,
                           long state_stride, const int* q_start, const int* seq_slots, void* out, hipStream_t stream);
+
+// ---- the gated delta rule with a decay per key channel (delta_rule.hip) ---------------------------------------------------
+// conv [tokens, conv_stride]: rows [q (groups x dim) | k (groups x dim) | v (heads x vdim)] after their convolutions and
+// activations; head h reads q / k number h / (heads / groups).  q, k -> unit vectors (x / sqrt(sum x^2 + unit_eps)), q times
+// q_scale; beta = sigmoid(beta_logits[t * beta_stride + h]); g = exp(-rate[h] * softplus(decay_logits[t, h, d] +
+// decay_bias[h, d])).  Per request and head, S [dim, vdim] (in the slot as [heads, vdim, dim] float32):
+// S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  out [tokens, heads x vdim] = o / rms(o) * norm_weight[i] *
+// sigmoid(gates[t, h, i]).  `workspace`: akv_delta_rule_workspace(...) floats.
+long akv_delta_rule_workspace(int tokens, int heads, int groups, int dim, int vdim);
+int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* beta_logits, long beta_stride,
+                   const float* decay_logits, const float* decay_bias, const float* rate, const float* gates,
+                   const float* norm_weight, float unit_eps, float norm_eps, float q_scale, float* state, long state_stride,
+                   const int* q_start, const int* seq_slots, float* workspace, void* out, int tokens, int seqs, int heads,
+                   int groups, int dim, int vdim, hipStream_t stream);
 
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
 // down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the

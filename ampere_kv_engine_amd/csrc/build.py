@@ -25,7 +25,7 @@ LIBRARY = "libakv_kernels.so"
 # a second library, compiled when a model first needs it: token-wise kernels, mixers and the routed feed-forward of
 # designs whose norms and residual sum are float32 throughout
 PARTS_SOURCES = ("tokenwise_f32.hip", "latent_attention.hip", "selective_scan.hip", "routed.hip", "gated_attention.hip",
-                 "recurrent_mixers.hip")
+                 "recurrent_mixers.hip", "delta_rule.hip")
 PARTS_HEADERS = ("common.h", "api_parts.h")
 PARTS_LIBRARY = "libakv_parts.so"
 ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library

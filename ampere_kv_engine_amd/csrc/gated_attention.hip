@@ -22,46 +22,76 @@ __device__ __forceinline__ void wave_sync_lds() {
 
 // One wave per (token, item): the token's query heads (normed into q_out), its key heads (normed into the token's slot
 // of the key pages) and its value heads (copied into the value pages).  projected rows: [q | k | v | ...].
+// With `maps` > 1 a head's queries and keys are `maps` vectors of `dim` side by side: the token has q_heads * maps query
+// vectors and kv_heads * maps key vectors, each normed and rotated for itself, and a key head's record in the pages is
+// its `maps` vectors one after the other.  With `table` [positions, rot_dims / 2, 2] (cos, sin) a vector's first rot_dims
+// dimensions are rotated by the token's position, dimension i with i + rot_dims / 2.
 template <typename T>
 __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restrict__ projected, long stride, long tokens,
                                                               int q_heads, int kv_heads, int dim, int vdim, float eps,
                                                               int normed, const int* __restrict__ slot_map,
                                                               T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
-                                                              long num_pages, T* __restrict__ q_out) {
+                                                              long num_pages, T* __restrict__ q_out, int maps,
+                                                              const float* __restrict__ table, int table_positions,
+                                                              int rot_dims, const int* __restrict__ positions) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  const int items = q_heads + 2 * kv_heads;
+  const int q_vectors = q_heads * maps, k_vectors = kv_heads * maps;
+  const int items = q_vectors + k_vectors + kv_heads;
   const long item = static_cast<long>(blockIdx.x) * waves + wave;
   if (item >= tokens * items) return;
   const long n = item / items;
   const int which = static_cast<int>(item % items);
   const T* row = projected + n * stride;
-  if (which < q_heads + kv_heads) {
-    const bool is_q = which < q_heads;
-    const T* x = row + static_cast<long>(which) * dim;       // (key heads follow the query heads at the same width)
+  if (which < q_vectors + k_vectors) {
+    const bool is_q = which < q_vectors;
+    const T* x = row + static_cast<long>(which) * dim;       // (key vectors follow the query vectors at the same width)
     T* y;
     if (is_q) {
-      y = q_out + (n * q_heads + which) * dim;
+      y = q_out + (n * q_vectors + which) * dim;
     } else {
       if (slot_map == nullptr) return;
       const long slot = slot_map[n];
       const long page = slot / page_size;
       if (slot < 0 || page >= num_pages) return;
-      y = k_pages + ((page * kv_heads + (which - q_heads)) * page_size + slot % page_size) * dim;
+      const int vector = which - q_vectors;
+      y = k_pages + (((page * kv_heads + vector / maps) * page_size + slot % page_size) * maps + vector % maps) * dim;
     }
-    float squares = 0.f;
-    for (int i = lane; i < dim; i += kWave) {
-      const float v = to_float(x[i]);
-      squares += v * v;
+    float scale = 1.f;
+    if (normed) {
+      float squares = 0.f;
+      for (int i = lane; i < dim; i += kWave) {
+        const float v = to_float(x[i]);
+        squares += v * v;
+      }
+      scale = rsqrtf(wave_sum(squares) / static_cast<float>(dim) + eps);
     }
-    const float scale = normed ? rsqrtf(wave_sum(squares) / static_cast<float>(dim) + eps) : 1.f;
-    for (int i = lane; i < dim; i += kWave) y[i] = from_float<T>(to_float(x[i]) * scale);
+    if (table == nullptr || rot_dims <= 0) {
+      for (int i = lane; i < dim; i += kWave) y[i] = from_float<T>(to_float(x[i]) * scale);
+    } else {
+      const int half = rot_dims / 2;
+      const int pos = positions[n];
+      const bool known = pos >= 0 && pos < table_positions;      // (a position beyond the table poisons the vector)
+      const float* angles = table + static_cast<long>(known ? pos : 0) * half * 2;
+      for (int i = lane; i < dim; i += kWave) {
+        float v = to_float(x[i]) * scale;
+        if (i < rot_dims) {
+          const bool low = i < half;
+          const int pair = low ? i : i - half;
+          const float c = angles[2 * pair], s = angles[2 * pair + 1];
+          const float other = to_float(x[low ? i + half : i - half]) * scale;
+          v = low ? v * c - other * s : v * c + other * s;
+          if (!known) v = __uint_as_float(0x7fc00000u);
+        }
+        y[i] = from_float<T>(v);
+      }
+    }
   } else {
     if (slot_map == nullptr) return;
-    const int h = which - q_heads - kv_heads;
+    const int h = which - q_vectors - k_vectors;
     const long slot = slot_map[n];
     const long page = slot / page_size;
     if (slot < 0 || page >= num_pages) return;
-    const T* x = row + static_cast<long>(q_heads + kv_heads) * dim + static_cast<long>(h) * vdim;
+    const T* x = row + static_cast<long>(q_vectors + k_vectors) * dim + static_cast<long>(h) * vdim;
     T* y = v_pages + (page * kv_heads + h) * vdim * page_size + slot % page_size;
     for (int i = lane; i < vdim; i += kWave) y[static_cast<long>(i) * page_size] = x[i];
   }
@@ -97,7 +127,9 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
     long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
     const int* __restrict__ block_table, const int* __restrict__ table_rows, int table_width, T* __restrict__ out,
     long tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-    int chunk, int window, int sink, long out_stride, float out_scale) {
+    int chunk, int window, int sink, long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps) {
+  // (`q_heads` counts query vectors: with `maps` > 1 a head has `maps` of them, which read the `maps` vectors of their key
+  // head's record in turn and the same values; vector v's key head is still v / (q_heads / kv_heads))
   extern __shared__ unsigned char lds_raw[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), kRowWaves = blockDim.x / kWave;
   // blocks go to the XCDs in turn: neighbouring rows - which read the same or neighbouring keys and values - are given to
@@ -123,10 +155,11 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
   __syncthreads();
 
   // with a sink the sums start as if a key of score 0 and no value had been seen (in the first wave's share)
+  // (a learned sink: the term is exp(sink_logits[head]) instead of exp(0))
   float m[G], l[G], acc[G][kMaxValueRegs];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    m[g] = sink && wave == 0 ? 0.f : -INFINITY;
+    m[g] = sink && wave == 0 ? (sink_logits != nullptr ? sink_logits[h0 + g] : 0.f) : -INFINITY;
     l[g] = sink && wave == 0 ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < kMaxValueRegs; ++c) acc[g][c] = 0.f;
@@ -144,7 +177,7 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
 #pragma unroll
         for (int g = 0; g < G; ++g) s[g] = __uint_as_float(0x7fc00000u);  // a page that is not the request's: poison
       } else {
-        const T* kp = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
+        const T* kp = k_pages + (((page * kv_heads + kvh) * page_size + j % page_size) * maps + h0 % maps) * dim;
         float dot[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) dot[g] = 0.f;
@@ -310,7 +343,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
     const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ block_table,
     const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, int first_row, int tokens, int q_heads,
     int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink,
-    long out_stride, float out_scale) {
+    long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps) {
   constexpr int DIM = 32 * DT, VDIM = 16 * VT;
   extern __shared__ float tile_shares[];      // [waves][2 + 4 VT][64]: what the block's waves found over their keys
   // a block is 16 rows and a head; its waves take the steps of 16 keys in turn
@@ -340,7 +373,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) qb[dt] = make_uint4(0u, 0u, 0u, 0u);
   }
-  float m = sink && wave == 0 ? 0.f : -INFINITY, l = sink && wave == 0 ? 1.f : 0.f;
+  float m = sink && wave == 0 ? (sink_logits != nullptr ? sink_logits[head] : 0.f) : -INFINITY, l = sink && wave == 0 ? 1.f : 0.f;
   const float inverse_cap = softcap > 0.f ? 1.f / softcap : 0.f;
   float4_t o[VT];
 #pragma unroll
@@ -363,7 +396,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
       const long page = block_table[table_at + j0 / page_size];
       if (page < 0 || page >= num_pages) return false;      // (uniform; a page that is not the request's is never read)
       const int o0 = j0 % page_size;
-      const bf16_t* kp = k_pages + ((page * kv_heads + kvh) * page_size + o0 + col) * DIM + grp * 8;
+      const bf16_t* kp = k_pages + (((page * kv_heads + kvh) * page_size + o0 + col) * maps + head % maps) * DIM + grp * 8;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) ks[dt] = load_bf16x8(kp + dt * 32);
       const bf16_t* vp = v_pages + ((page * kv_heads + kvh) * VDIM + col) * page_size + o0 + grp * 4;
@@ -492,9 +525,9 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
                               float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
-                              hipStream_t stream) {
+                              const float* sink_logits, int maps, hipStream_t stream) {
   if (tokens <= first_row) return 0;
-  if (page_size % 16 != 0 || q_heads % kv_heads != 0) return -2;
+  if (page_size % 16 != 0 || q_heads % kv_heads != 0 || maps < 1) return -2;
   const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
   const unsigned grid = static_cast<unsigned>(((tokens - first_row + 15) / 16 + kXcds - 1) / kXcds * kXcds * q_heads);
   const int waves = vdim > 128 ? 2 : 4;       // (their shares must fit into 64 KB of LDS)
@@ -504,7 +537,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages),         \
       static_cast<const bf16_t*>(gates), gate_stride, gate_at, seq_of_token, q_start, positions, block_table, table_rows, \
       table_width, static_cast<bf16_t*>(out), first_row, tokens, q_heads, kv_heads, page_size, num_pages, scale, softcap, \
-      chunk, window, sink, out_stride, out_scale)
+      chunk, window, sink, out_stride, out_scale, sink_logits, maps)
 #define AKV_TILES_V(DT)                    \
   switch (vdim) {                          \
     case 32: AKV_TILES(DT, 2); break;      \
@@ -527,14 +560,16 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
 
 int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
                         int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
-                        long num_pages, void* q_out, hipStream_t stream) {
+                        long num_pages, void* q_out, int maps, const float* table, int table_positions, int rot_dims,
+                        const int* positions, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0) return -2;
-  const long items = tokens * (q_heads + 2 * kv_heads);
+  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || maps < 1) return -2;
+  if (table != nullptr && (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > dim || positions == nullptr)) return -2;
+  const long items = tokens * ((q_heads + kv_heads) * maps + kv_heads);
   AKV_DISPATCH(dtype, T, unit_norm_write_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(
                              static_cast<const T*>(projected), stride, tokens, q_heads, kv_heads, dim, vdim, eps, normed,
                              slot_map, static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages,
-                             static_cast<T*>(q_out)));
+                             static_cast<T*>(q_out), maps, table, table_positions, rot_dims, positions));
   return AKV_LAUNCH_STATUS();
 }
 
@@ -543,8 +578,9 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
                              int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
-                             hipStream_t stream) {
+                             const float* sink_logits, int maps, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (maps < 1) return -2;
   const int kRowWaves = row_waves;
   if (row_waves < 1 || row_waves > kMaxRowWaves) return -2;
   if (vdim > kMaxValueRegs * kWave || dim <= 0 || q_heads % kv_heads != 0) return -2;
@@ -574,7 +610,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                    static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),            \
                    static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows, \
                    table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale, \
-                   softcap, chunk, window, sink, out_stride, out_scale))
+                   softcap, chunk, window, sink, out_stride, out_scale, sink_logits, maps))
 #define AKV_ROWS_G(VEC)          \
   switch (bundle) {              \
     case 4: AKV_ROWS(VEC, 4); break; \

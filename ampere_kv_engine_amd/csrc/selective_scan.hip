@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ x,
   const int r = seq_of_token[n];
   const int first = q_start[r];
   const float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + conv_at;   // [taps - 1][channels]
-  float acc = to_float(bias[c]);
+  float acc = bias != nullptr ? to_float(bias[c]) : 0.f;
   for (int k = 0; k < taps; ++k) {
     const int row = n - (taps - 1 - k);
     float v;

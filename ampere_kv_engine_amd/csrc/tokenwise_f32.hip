@@ -77,7 +77,8 @@ template <typename T, int GROUPS>
 __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                                  const float* __restrict__ post_weight, float post_eps,
                                                                  const float* __restrict__ pre_weight, float pre_eps,
-                                                                 T* __restrict__ out, int hidden, float delta_scale) {
+                                                                 T* __restrict__ out, int hidden, float delta_scale,
+                                                                 const float* __restrict__ offset) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float4 kept[GROUPS], added[GROUPS];
@@ -111,6 +112,16 @@ __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restri
         d = make_float4(d.x * delta_scale, d.y * delta_scale, d.z * delta_scale, d.w * delta_scale);
       }
       kept[j] = make_float4(kept[j].x + d.x, kept[j].y + d.y, kept[j].z + d.z, kept[j].w + d.w);
+      if (offset == nullptr) write4<float>(stream + base + i, kept[j]);
+    }
+  }
+  if (offset != nullptr) {      // the same vector on every row, after the branch
+#pragma unroll
+    for (int j = 0; j < GROUPS; ++j) {
+      const int i = (j * 256 + static_cast<int>(threadIdx.x)) * 4;
+      if (i >= hidden) continue;
+      const float4 b = read4<float>(offset + i);
+      kept[j] = make_float4(kept[j].x + b.x, kept[j].y + b.y, kept[j].z + b.z, kept[j].w + b.w);
       write4<float>(stream + base + i, kept[j]);
     }
   }
@@ -133,26 +144,31 @@ template <typename T>
 __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                             const float* __restrict__ post_weight, float post_eps,
                                                             const float* __restrict__ pre_weight, float pre_eps,
-                                                            T* __restrict__ out, int hidden, float delta_scale) {
+                                                            T* __restrict__ out, int hidden, float delta_scale,
+                                                            const float* __restrict__ offset) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float* s = stream + base;
   float squares = 0.f;
-  if (delta != nullptr) {
-    const T* d = delta + base;
-    float post_scale = 1.f;
-    if (post_weight != nullptr) {
-      float acc = 0.f;
-      for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-        const float v = to_float(d[i]);
-        acc += v * v;
+  if (delta != nullptr || offset != nullptr) {
+    // (a thread meets the same elements in every pass: it reads back what it wrote itself)
+    if (delta != nullptr) {
+      const T* d = delta + base;
+      float post_scale = 1.f;
+      if (post_weight != nullptr) {
+        float acc = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+          const float v = to_float(d[i]);
+          acc += v * v;
+        }
+        post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
       }
-      post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
+      for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+        s[i] += post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]) * delta_scale;
     }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float add = post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]) * delta_scale;
-      const float v = s[i] + add;
-      s[i] = v;
+      const float v = offset != nullptr ? s[i] + offset[i] : s[i];
+      if (offset != nullptr) s[i] = v;
       squares += v * v;
     }
   } else if (out != nullptr) {
@@ -166,6 +182,80 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ 
   T* o = out + base;
   // (a thread reads back what it wrote itself: the same elements in every pass)
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(s[i] * scale * pre_weight[i]);
+}
+
+// ---- embedding followed by a norm: out = table[id] / rms(table[id]) * weight, float32 --------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void embed_normed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                                           const float* __restrict__ weight, float eps,
+                                                           float* __restrict__ out, int hidden, int vocab,
+                                                           const int* __restrict__ seq_of_token,
+                                                           const int* __restrict__ seq_slots,
+                                                           const int* __restrict__ slot_words) {
+  __shared__ float scratch[16];
+  const int n = blockIdx.x;
+  int id = ids[n];
+  if (id == -1 && slot_words != nullptr)
+    id = slot_words[static_cast<long>(seq_slots[seq_of_token[n]]) * kSlotWords + kSlotLastToken];
+  float* dst = out + static_cast<size_t>(n) * hidden;
+  if (id < 0 || id >= vocab) {     // never read outside the table; a poisoned row shows the fault downstream
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = __uint_as_float(kPoison);
+    return;
+  }
+  const T* row = table + static_cast<size_t>(id) * hidden;
+  float squares = 0.f;
+  for (int d = threadIdx.x; d < hidden; d += blockDim.x) {
+    const float v = to_float(row[d]);
+    squares += v * v;
+  }
+  const float scale = rsqrtf(block_sum(squares, scratch) / static_cast<float>(hidden) + eps);
+  for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(row[d]) * scale * weight[d];
+}
+
+// ---- a gated feed-forward's activation after a stacked product: out = act(gate) * up --------------------------------------
+__device__ __forceinline__ float gelu_tanh_of(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long tokens, int inter,
+                                        int activation) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= tokens * inter) return;
+  const long n = index / inter;
+  const int i = static_cast<int>(index % inter);
+  const float gate = to_float(gate_up[n * 2 * inter + i]), up = to_float(gate_up[n * 2 * inter + inter + i]);
+  const float act = activation == 1 ? gelu_tanh_of(gate) : gate / (1.f + expf(-gate));
+  out[index] = from_float<T>(act * up);
+}
+
+// ---- the difference of two attention maps, normed and gated ------------------------------------------------------------
+// maps [tokens, heads, 2, vdim]: o = a1 - lambda a2; o / rms(o) * after; times sigmoid(gates[t, gate_at + h * vdim + i]).
+// One wave per (token, head); lambda is read on the device.
+template <typename T>
+__global__ __launch_bounds__(256) void difference_norm_gate_kernel(const T* __restrict__ maps, const float* __restrict__ lambda,
+                                                                   float eps, float after, const T* __restrict__ gates,
+                                                                   long gate_stride, long gate_at, T* __restrict__ out,
+                                                                   long items, int heads, int vdim) {
+  const long item = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  if (item >= items) return;
+  const long n = item / heads;
+  const int h = static_cast<int>(item % heads);
+  const T* first = maps + item * 2 * vdim;
+  const T* second = first + vdim;
+  const float lam = lambda[0];
+  float squares = 0.f;
+  for (int i = lane; i < vdim; i += kWave) {
+    const float o = to_float(first[i]) - lam * to_float(second[i]);
+    squares = fmaf(o, o, squares);
+  }
+  const float scale = rsqrtf(wave_sum(squares) / static_cast<float>(vdim) + eps) * after;
+  for (int i = lane; i < vdim; i += kWave) {
+    const float o = to_float(first[i]) - lam * to_float(second[i]);
+    const float gate = 1.f / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + static_cast<long>(h) * vdim + i])));
+    out[item * vdim + i] = from_float<T>(o * scale * gate);
+  }
 }
 
 // out = a * scale_a + b * scale_b, formed in float32 and rounded once (out may be a or b).
@@ -184,6 +274,37 @@ int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, v
   if (count <= 0) return 0;
   AKV_DISPATCH(dtype, T, scaled_sum_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
                              static_cast<const T*>(a), scale_a, static_cast<const T*>(b), scale_b, static_cast<T*>(out), count));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_embed_normed(const int* ids, const void* table, int dtype, const float* weight, float eps, float* out, int tokens,
+                     int hidden, int vocab, const int* seq_of_token, const int* seq_slots, const int* slot_words,
+                     hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(dtype, T, embed_normed_kernel<T><<<tokens, 256, 0, stream>>>(ids, static_cast<const T*>(table), weight, eps,
+                                                                            out, hidden, vocab, seq_of_token, seq_slots,
+                                                                            slot_words));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_gated_activation(const void* gate_up, void* out, int dtype, long tokens, int inter, int activation,
+                         hipStream_t stream) {
+  if (tokens <= 0 || inter <= 0) return 0;
+  if (activation != 0 && activation != 1) return -2;
+  const long count = tokens * inter;
+  AKV_DISPATCH(dtype, T, gated_activation_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
+                             static_cast<const T*>(gate_up), static_cast<T*>(out), tokens, inter, activation));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_difference_norm_gate(const void* maps, const float* lambda, float eps, float after, const void* gates,
+                             long gate_stride, long gate_at, void* out, int dtype, long tokens, int heads, int vdim,
+                             hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  const long items = tokens * heads;
+  AKV_DISPATCH(dtype, T, difference_norm_gate_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(
+                             static_cast<const T*>(maps), lambda, eps, after, static_cast<const T*>(gates), gate_stride,
+                             gate_at, static_cast<T*>(out), items, heads, vdim));
   return AKV_LAUNCH_STATUS();
 }
 
@@ -214,10 +335,10 @@ int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots
 
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      float delta_scale, hipStream_t stream) {
+                      float delta_scale, const float* offset, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (out != nullptr && pre_weight == nullptr) return -2;
-#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden, delta_scale
+#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden, delta_scale, offset
   AKV_DISPATCH(dtype, T, {
     if (hidden % 4 == 0 && hidden >= 4 && hidden <= 256 * 4 * 2) norm_add_norm_rows_kernel<T, 2><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
     else if (hidden % 4 == 0 && hidden <= 256 * 4 * 8) norm_add_norm_rows_kernel<T, 8><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);

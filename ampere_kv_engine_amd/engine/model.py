@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelSpec
-from ..parts.base import PagedKV, Runtime, SlotState, StreamSums, Unsettled, build_part
+from ..parts.base import PagedKV, Runtime, ScaledDelta, SlotState, StreamSums, Unsettled, build_part
 from ..weights.spec import TensorSpec
 
 
@@ -35,6 +35,8 @@ class Model:
         self.spec, self.rt = spec, runtime
         self.embedding, self.blocks, self.final_norm, self.head = _assemble(spec, runtime)
         self.final_norm_name = spec.final_norm.get("name", "model.norm.weight")
+        # vectors that run-order entries add to the residual sum before they run (a pass over repeated layers)
+        self.pass_vectors = build_part("embedding", spec.pass_vectors, runtime) if spec.pass_vectors is not None else None
 
     # ---- weights ----------------------------------------------------------------------------------
     def tensors(self) -> list[TensorSpec]:
@@ -43,6 +45,8 @@ class Model:
             specs += block.tensors(layer.prefix)
         specs += self.final_norm.tensors(self.final_norm_name)
         specs += self.head.tensors()
+        if self.pass_vectors is not None:
+            specs += self.pass_vectors.tensors()
         tied = self.spec.head.get("tied_to")
         if tied is not None:
             # a file of a tied model may still carry the head's tensor; it must then hold the embedding's values
@@ -56,17 +60,21 @@ class Model:
         for layer, block in zip(self.spec.layers, self.blocks):
             block.load(fetch, layer.prefix)
         self.final_norm.load(fetch, self.final_norm_name)
+        if self.pass_vectors is not None:
+            self.pass_vectors.load(fetch)
         if self.spec.head.get("tied_to") is not None:
             self.head.load(fetch, tied_weight=self.embedding.weight)
         else:
             self.head.load(fetch)
 
     def cache_needs(self) -> dict[int, PagedKV | SlotState | None]:
-        """What each cache layer keeps between steps, asked of the mixer of the layer that owns it."""
+        """What each cache keeps between steps, asked of the mixer of the layer that owns it (a layer that runs several
+        times, each time with a cache of its own, is asked once per copy)."""
         needs = {}
         for entry in self.spec.run_order:
-            if entry.cache_layer not in needs:
-                needs[entry.cache_layer] = self.blocks[entry.cache_layer].mixer.cache_request()
+            key = self.spec.cache_key(entry)
+            if key not in needs:
+                needs[key] = self.blocks[entry.cache_layer].mixer.cache_request()
         return needs
 
     def weight_bytes_per_step(self) -> int:
@@ -98,10 +106,12 @@ class Model:
             following = self.blocks[order[step_index + 1].layer] if step_index + 1 < len(order) else None
             ctx.fold_into_stream = following is None or following.takes_stream_sums
             ctx.fold_gain = following.entry_gain() if following is not None and following.takes_stream_sums else None
+            if entry.adds_row is not None:
+                pending = self._with_vector(pending, self.pass_vectors.row(entry.adds_row), ctx)
             if isinstance(pending, Unsettled) and not self.blocks[entry.layer].takes_normed_delta:
                 pending.settle(ctx.stream)       # the reader knows tensors only: the branch is normed and added first
                 pending = None
-            pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
+            pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[self.spec.cache_key(entry)],
                                                        entry.writes_cache)
         if isinstance(pending, StreamSums):      # the last branch's output is in the residual sum already
             pending = None
@@ -121,6 +131,22 @@ class Model:
         if logits_out is None:
             logits_out = torch.empty((wanted, self.spec.vocab_size), dtype=torch.float32, device=rt.device)
         return self.head.forward(normed, logits_out)
+
+
+    def _with_vector(self, pending, vector, ctx):
+        """`pending` with `vector` still to be added to every row of the residual sum after it: a branch that is added
+        times a constant takes the vector along into the kernel that adds it; anything else is settled first."""
+        k = self.rt.kernels
+        if isinstance(pending, ScaledDelta) and pending.offset is None:
+            return ScaledDelta(pending.delta, pending.scale, k, offset=vector)
+        if isinstance(pending, Unsettled):
+            pending.settle(ctx.stream)
+            pending = None
+        if pending is None:
+            return ScaledDelta(None, 1.0, k, offset=vector)
+        if isinstance(pending, StreamSums):
+            raise TypeError("a vector cannot follow a branch that has left only its rows' sums of squares")
+        return ScaledDelta(pending, 1.0, k, offset=vector)
 
 
 def expected_tensors(spec: ModelSpec) -> list[TensorSpec]:

@@ -46,8 +46,10 @@ class PartsKernels:
                          "akv_conv_state_update", "akv_selective_scan", "akv_route", "akv_gate_relu_squared",
                          "akv_parts_slot_layout", "akv_conv_taps", "akv_scaled_sum", "akv_unit_norm_write",
                          "akv_gated_attention_rows", "akv_gated_attention_tiles", "akv_retention", "akv_retention_chunked", "akv_gated_linear_scan", "akv_route_chosen",
-                         "akv_gate_silu_mul"):
+                         "akv_gate_silu_mul", "akv_embed_normed", "akv_gated_activation", "akv_difference_norm_gate",
+                         "akv_delta_rule"):
                 getattr(lib, name).restype = ctypes.c_int
+            lib.akv_delta_rule_workspace.restype = ctypes.c_long
             layout = (ctypes.c_int * 3)()
             lib.akv_parts_slot_layout(layout)
             if tuple(layout) != (slots.SLOT_WORDS, slots.WORD_LAST_TOKEN, slots.WORD_FED_TOKEN):
@@ -101,10 +103,11 @@ class PartsKernels:
         self._check(lib.akv_note_fed_tokens(_ptr(ids), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(words), ctx.num_seqs,
                                             self._stream()), "note_fed_tokens")
 
-    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale: float = 1.0) -> None:
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale: float = 1.0,
+                      offset=None) -> None:
         """stream (float32) += delta / rms(delta) * post_weight (+= delta_scale * delta where `post_weight` is None; nothing
-        where `delta` is None); then, where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one
-        rounding of a stored result."""
+        where `delta` is None); then stream += offset (a float32 vector, the same on every row) where there is one; then,
+        where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one rounding of a stored result."""
         tokens, hidden = stream.shape
         self._dense(stream, "stream", torch.float32)
         dtype = None
@@ -117,12 +120,63 @@ class PartsKernels:
             dtype = out.dtype
         if post_weight is not None:
             self._dense(post_weight, "post_weight", torch.float32, (hidden,))
+        if offset is not None:
+            self._dense(offset, "offset", torch.float32, (hidden,))
+            dtype = dtype or torch.float32
         if dtype is None:
             return
         self._check(self._parts().akv_norm_add_norm(_ptr(stream), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps),
                                                     _ptr(pre_weight), ctypes.c_float(pre_eps), _ptr(out), _DTYPE_CODE[dtype],
-                                                    tokens, hidden, ctypes.c_float(delta_scale), self._stream()),
+                                                    tokens, hidden, ctypes.c_float(delta_scale), _ptr(offset), self._stream()),
                     "norm_add_norm")
+
+    def embed_normed(self, ids, table, weight, eps: float, out, ctx=None) -> None:
+        """out[n] = table[id] / rms(table[id]) * weight, float32: an embedding whose rows are normed before the first layer.
+        With the step's context an id of -1 is the token chosen last for the row's request."""
+        tokens = ids.shape[0]
+        self._dense(ids, "ids", torch.int32, (tokens,))
+        self._dense(table, "table")
+        vocab, hidden = table.shape
+        self._dense(weight, "weight", torch.float32, (hidden,))
+        self._dense(out, "out", torch.float32, (tokens, hidden))
+        words = getattr(ctx, "slot_words", None) if ctx is not None else None
+        seq_of_token = seq_slots = None
+        if words is not None:
+            seq_of_token, seq_slots = ctx.seq_of_token, ctx.seq_slots
+            self._dense(words, "slot_words", torch.int32)
+            self._dense(seq_of_token, "seq_of_token", torch.int32, (tokens,))
+            self._dense(seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+            if max(ctx.host_seq_slots) >= words.shape[0]:
+                self._refuse("a request's slot lies outside the slot words")
+        self._check(self._parts().akv_embed_normed(_ptr(ids), _ptr(table), self._code_of(table), _ptr(weight),
+                                                   ctypes.c_float(eps), _ptr(out), tokens, hidden, vocab, _ptr(seq_of_token),
+                                                   _ptr(seq_slots), _ptr(words), self._stream()), "embed_normed")
+
+    GATED_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+    def gated_activation(self, gate_up, out, activation: str) -> None:
+        """out [tokens, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:], in float32 with one rounding."""
+        tokens, inter = out.shape
+        self._dense(out, "out")
+        self._dense(gate_up, "gate_up", out.dtype, (tokens, 2 * inter))
+        if activation not in self.GATED_ACTIVATIONS:
+            self._refuse(f"a gated feed-forward's activation is one of {sorted(self.GATED_ACTIVATIONS)}, not {activation!r}")
+        self._check(self._parts().akv_gated_activation(_ptr(gate_up), _ptr(out), self._code_of(out), _long(tokens), inter,
+                                                       self.GATED_ACTIVATIONS[activation], self._stream()), "gated_activation")
+
+    def difference_norm_gate(self, maps, lam, eps: float, after: float, gates, gate_at: int, heads: int, vdim: int, out) -> None:
+        """maps [tokens, heads * 2 * vdim] (per head: map 1, map 2) -> out [tokens, heads * vdim] = (a1 - lam a2) /
+        rms(a1 - lam a2) * after * sigmoid(gates[:, gate_at + h * vdim + i]); `lam`: one float32 on the device."""
+        tokens = maps.shape[0]
+        self._dense(maps, "maps", None, (tokens, heads * 2 * vdim))
+        self._dense(out, "out", maps.dtype, (tokens, heads * vdim))
+        self._dense(lam, "lam", torch.float32, (1,))
+        self._dense(gates, "gates", maps.dtype)
+        if gates.dim() != 2 or gates.shape[0] != tokens or gate_at < 0 or gate_at + heads * vdim > gates.shape[1]:
+            self._refuse(f"gates must be [tokens, at least {gate_at + heads * vdim}], got {tuple(gates.shape)}")
+        self._check(self._parts().akv_difference_norm_gate(
+            _ptr(maps), _ptr(lam), ctypes.c_float(eps), ctypes.c_float(after), _ptr(gates), _long(gates.shape[1]),
+            _long(gate_at), _ptr(out), self._code_of(maps), _long(tokens), heads, vdim, self._stream()), "difference_norm_gate")
 
     def scaled_sum(self, a, scale_a: float, b, scale_b: float, out) -> None:
         """out = a * scale_a + b * scale_b, in float32 with one rounding (`out` may be `a` or `b`)."""
@@ -304,29 +358,93 @@ class PartsKernels:
         if max(ctx.host_seq_slots) >= state.shape[0]:
             self._refuse("a request's slot lies outside the state")
 
-    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation: str = "silu") -> None:
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation: str = "silu", conv_at=None) -> None:
         """out[t, c] = silu(bias[c] + sum_k weight[c, k] * x[t - (taps - 1 - k), c]) over the first `channels` columns
-        of `xz` (with `activation="none"` the sum as it is); inputs before a portion come from the request's state (zeros before its first token).  Afterwards the
-        state holds the last taps - 1 inputs of every request of the step."""
+        of `xz` (with `activation="none"` the sum as it is; `bias` None: none); inputs before a portion come from the
+        request's state (zeros before its first token).  Afterwards the state holds the last taps - 1 inputs of every
+        request of the step.  The inputs lie in the state from element `conv_at` on (default: after `channels * n_state`
+        elements, and the state holds nothing else)."""
         tokens, taps = xz.shape[0], weight.shape[1]
         self._dense(xz, "xz")
         if xz.dim() != 2 or xz.shape[1] < channels:
             self._refuse(f"xz must be [tokens, at least {channels}], got {tuple(xz.shape)}")
         self._dense(weight, "weight", None, (channels, taps))
-        self._dense(bias, "bias", weight.dtype, (channels,))
+        if bias is not None:
+            self._dense(bias, "bias", weight.dtype, (channels,))
         self._dense(out, "out", xz.dtype, (tokens, channels))
-        self._scan_state(state, ctx, channels, n_state, taps)
+        if conv_at is None:
+            self._scan_state(state, ctx, channels, n_state, taps)
+            conv_at = channels * n_state
+        else:
+            self._dense(state, "state", torch.float32)
+            if state.dim() != 2 or conv_at < 0 or state.shape[1] < conv_at + (taps - 1) * channels:
+                self._refuse(f"the state must hold {(taps - 1) * channels} inputs from element {conv_at} on, got {tuple(state.shape)}")
+            if max(ctx.host_seq_slots) >= state.shape[0]:
+                self._refuse("a request's slot lies outside the state")
         self._step_arrays(ctx, tokens)
-        lib, conv_at = self._parts(), channels * n_state
+        lib = self._parts()
         if activation not in ("silu", "none"):
             self._refuse(f"the convolution's activation is 'silu' or 'none', not {activation!r}")
         self._check(lib.akv_conv_taps(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(weight), _ptr(bias),
                                       self._code_of(weight), _ptr(state), _long(state.shape[1]), _long(conv_at),
                                       _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), tokens,
                                       channels, taps, 1 if activation == "silu" else 0, self._stream()), "conv_taps")
-        self._check(lib.akv_conv_state_update(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(state),
-                                              _long(state.shape[1]), _long(conv_at), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
-                                              ctx.num_seqs, channels, taps, self._stream()), "conv_state_update")
+        if taps > 1:
+            self._check(lib.akv_conv_state_update(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(state),
+                                                  _long(state.shape[1]), _long(conv_at), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
+                                                  ctx.num_seqs, channels, taps, self._stream()), "conv_state_update")
+
+    # ---- the gated delta rule --------------------------------------------------------------------------------------------
+    def check_delta_rule_sizes(self, heads: int, groups: int, dim: int, vdim: int) -> None:
+        if heads % groups or not 0 < dim <= 2048 or vdim <= 0:
+            self._refuse(f"the delta rule takes heads that are a multiple of the key heads and keys up to 2048 wide, not "
+                         f"{heads} / {groups} heads of {dim}")
+
+    def delta_rule(self, conv, beta_logits, beta_at: int, decay_logits, decay_bias, rate, gates, norm_weight, unit_eps: float,
+                   norm_eps: float, q_scale: float, heads: int, groups: int, dim: int, vdim: int, state, ctx, out) -> None:
+        """conv [tokens, 2 * groups * dim + heads * vdim]: q, k and v after their convolutions and activations.  q and k
+        become unit vectors per head (x / sqrt(sum x^2 + unit_eps); q times q_scale); beta = sigmoid(beta_logits[:, beta_at +
+        h]); g = exp(-rate[h] * softplus(decay_logits[t, h, d] + decay_bias[h, d])).  Per request and head, token after
+        token: S <- g S (rows are key channels); u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  out [tokens, heads * vdim]
+        = o / rms(o) * norm_weight * sigmoid(gates).  S lies at the start of the request's slot of `state`, float32, as
+        [heads, vdim, dim]."""
+        tokens = conv.shape[0]
+        width = 2 * groups * dim + heads * vdim
+        self._dense(conv, "conv", None, (tokens, width))
+        self._dense(beta_logits, "beta_logits", conv.dtype)
+        if beta_logits.dim() != 2 or beta_logits.shape[0] != tokens or beta_at < 0 or beta_at + heads > beta_logits.shape[1]:
+            self._refuse(f"beta_logits must be [tokens, at least {beta_at + heads}], got {tuple(beta_logits.shape)}")
+        self._dense(decay_logits, "decay_logits", torch.float32, (tokens, heads * dim))
+        self._dense(decay_bias, "decay_bias", torch.float32, (heads * dim,))
+        self._dense(rate, "rate", torch.float32, (heads,))
+        self._dense(gates, "gates", torch.float32, (tokens, heads * vdim))
+        self._dense(norm_weight, "norm_weight", torch.float32, (vdim,))
+        self._dense(out, "out", conv.dtype, (tokens, heads * vdim))
+        self._dense(state, "state", torch.float32)
+        if state.dim() != 2 or state.shape[1] < heads * dim * vdim:
+            self._refuse(f"the state must be [slots, at least {heads * dim * vdim}], got {tuple(state.shape)}")
+        if max(ctx.host_seq_slots) >= state.shape[0]:
+            self._refuse("a request's slot lies outside the state")
+        self.check_delta_rule_sizes(heads, groups, dim, vdim)
+        self._step_arrays(ctx, tokens)
+        lib = self._parts()
+        workspace = self._delta_workspace(int(lib.akv_delta_rule_workspace(tokens, heads, groups, dim, vdim)))
+        self._check(lib.akv_delta_rule(
+            _ptr(conv), _long(width), self._code_of(conv), _ptr_at(beta_logits, beta_at), _long(beta_logits.shape[1]),
+            _ptr(decay_logits), _ptr(decay_bias), _ptr(rate), _ptr(gates), _ptr(norm_weight), ctypes.c_float(unit_eps),
+            ctypes.c_float(norm_eps), ctypes.c_float(q_scale), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start),
+            _ptr(ctx.seq_slots), _ptr(workspace), _ptr(out), tokens, ctx.num_seqs, heads, groups, dim, vdim, self._stream()),
+            "delta_rule")
+
+    def _delta_workspace(self, need: int) -> torch.Tensor:
+        """Where the tokens' unit vectors, decays and raw outputs lie during a step."""
+        held = self.__dict__.get("_delta_buffer")
+        if held is None or held.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                self._refuse("a recorded step needs more room for the delta rule's tokens than the steps before it")
+            self.__dict__.setdefault("_delta_outgrown", []).append(held)
+            held = self.__dict__["_delta_buffer"] = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=self.device)
+        return held
 
     def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out) -> None:
         """Per request and channel, token after token: S <- exp(softplus(dt) A) S + softplus(dt) x B, y = S C + D x,
@@ -409,34 +527,60 @@ class PartsKernels:
         self._dense(v_pages, "v_pages", dtype, (k_pages.shape[0], kv_heads, vdim, k_pages.shape[2]))
         return k_pages.shape[0], k_pages.shape[2]
 
-    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at: int = 0) -> None:
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at: int = 0,
+                        maps: int = 1, table=None, rot_dims: int = 0, positions=None) -> None:
         """projected [tokens, ... | q | k | v | ...] with q at column `at`: the query heads divided by their root mean square (eps inside the root;
         `eps` None: as they are) -> q_out; with `slot_map` the key heads, the same way, and the value heads into the
-        tokens' slots of the pages."""
+        tokens' slots of the pages.  `maps` > 1: a head's queries and keys are `maps` vectors of `dim` side by side, each
+        normed and rotated for itself; a key head's record in the pages is `maps * dim` wide.  `table` [positions,
+        rot_dims / 2, 2] (cos, sin): every vector's first `rot_dims` dimensions are rotated by the token's position
+        (`positions`), dimension i with i + rot_dims / 2, after the norm."""
         tokens = projected.shape[0]
         self._dense(projected, "projected")
-        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + (q_heads + kv_heads) * dim + kv_heads * vdim:
+        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + (q_heads + kv_heads) * maps * dim + kv_heads * vdim:
             self._refuse(f"projected rows must hold queries, keys and values, got {tuple(projected.shape)}")
-        self._dense(q_out, "q_out", projected.dtype, (tokens, q_heads * dim))
-        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, projected.dtype)
+        self._dense(q_out, "q_out", projected.dtype, (tokens, q_heads * maps * dim))
+        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, maps * dim, vdim, projected.dtype)
         if slot_map is not None:
             self._dense(slot_map, "slot_map", torch.int32, (tokens,))
+        table_positions = 0
+        if table is not None:
+            self._dense(table, "table", torch.float32)
+            if rot_dims <= 0 or rot_dims % 2 or rot_dims > dim or table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
+                self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2] for an even rot_dims of at most {dim}, "
+                             f"got {tuple(table.shape)} for {rot_dims}")
+            self._dense(positions, "positions", torch.int32, (tokens,))
+            table_positions = table.shape[0]
         self._check(self._parts().akv_unit_norm_write(
             _ptr_at(projected, at), _long(projected.shape[1]), self._code_of(projected), _long(tokens), q_heads, kv_heads, dim,
             vdim, ctypes.c_float(eps if eps is not None else 0.0), 0 if eps is None else 1, _ptr(slot_map), _ptr(k_pages),
-            _ptr(v_pages), page_size, _long(num_pages), _ptr(q_out), self._stream()), "unit_norm_write")
+            _ptr(v_pages), page_size, _long(num_pages), _ptr(q_out), maps, _ptr(table), table_positions,
+            rot_dims if table is not None else 0, _ptr(positions) if table is not None else ctypes.c_void_p(0),
+            self._stream()), "unit_norm_write")
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
-                        chunk, window, sink, out, out_at: int = 0, out_scale: float = 1.0) -> None:
+                        chunk, window, sink, out, out_at: int = 0, out_scale: float = 1.0, sink_logits=None,
+                        maps: int = 1) -> None:
         """Every query head attends the keys of its request that it sees (see `parts/gated_attention.py`) -> columns
         out_at .. out_at + q_heads * vdim of `out`, times `out_scale`; `gates` [tokens, width]: head h's output times
-        sigmoid(gates[t, gate_at + h])."""
+        sigmoid(gates[t, gate_at + h]).  `sink_logits` [q_heads] float32 (with `sink`): the denominator's extra term is
+        exp(sink_logits[h]) instead of exp(0).  `maps` > 1: a head has `maps` query vectors, each an attention of its own
+        over the vector of the same number in its key head's record ([pages, kv_heads, page, maps * dim]) and over the
+        head's values; out then holds q_heads * maps outputs a token, a head's maps side by side."""
         tokens = q.shape[0]
+        heads = q_heads
+        q_heads = heads * maps          # (from here on: query vectors)
         self._dense(q, "q", None, (tokens, q_heads * dim))
         self._dense(out, "out", q.dtype)
         if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + q_heads * vdim > out.shape[1]:
             self._refuse(f"out must be [tokens, at least {out_at + q_heads * vdim}], got {tuple(out.shape)}")
-        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, q.dtype)
+        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, maps * dim, vdim, q.dtype)
+        if maps > 1 and gates is not None:
+            self._refuse("a gate per head and several maps per head do not go together")
+        if sink_logits is not None:
+            self._dense(sink_logits, "sink_logits", torch.float32, (q_heads,))
+            if not sink:
+                self._refuse("sink logits without a sink")
         gate_stride = 0
         if gates is not None:
             self._dense(gates, "gates", q.dtype)
@@ -457,7 +601,7 @@ class PartsKernels:
             self._refuse("a request is longer than its row of the block table")
         tail = (ctypes.c_float(scale), ctypes.c_float(softcap if softcap is not None else 0.0),
                 int(chunk) if chunk is not None else 0, int(window) if window is not None else 0, 1 if sink else 0,
-                _long(out.shape[1]), ctypes.c_float(out_scale), self._stream())
+                _long(out.shape[1]), ctypes.c_float(out_scale), _ptr(sink_logits), maps, self._stream())
         singles = tokens
         if (q.dtype == torch.bfloat16 and dim in self.MATRIX_CORE_HEAD_DIMS and vdim in self.MATRIX_CORE_HEAD_DIMS
                 and page_size % 16 == 0 and out.shape[1] % 4 == 0 and out_at % 4 == 0):
@@ -476,8 +620,8 @@ class PartsKernels:
             self._check(self._parts().akv_gated_attention_rows(
                 _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
                 _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr_at(out, out_at),
-                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail[:-1], row_waves,
-                tail[-1]), "gated_attention")
+                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail[:-3], row_waves,
+                *tail[-3:]), "gated_attention")
 
     # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
     def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:

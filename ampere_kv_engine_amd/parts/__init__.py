@@ -1,9 +1,12 @@
 from .base import (CATEGORIES, KernelSet, Norm, NormedDelta, PagedKV, Part, Runtime, SlotState, StreamSums, UnnormedRows, build_part,
                    register_part, registered)
 from . import (norm, position, linear, feed_forward, attention, block, embedding, latent_attention,  # noqa: F401
-               selective_scan, routed_experts, gated_attention, retention, parallel, rglru)      # (registers the kinds)
+               selective_scan, routed_experts, gated_attention, retention, parallel, rglru,      # (registers the kinds)
+               differential_attention, delta_rule)
 from .attention import Attention
 from .block import NoFeedForward, PreNormBlock, SandwichBlock, ScaledPreNormBlock
+from .delta_rule import GatedDeltaRule
+from .differential_attention import DifferentialAttention
 from .gated_attention import GatedAttention
 from .parallel import ParallelMixers
 from .retention import Retention
@@ -19,7 +22,7 @@ from .position import NoPosition, RotaryHalf
 
 __all__ = ["CATEGORIES", "KernelSet", "Norm", "PagedKV", "Part", "Runtime", "SlotState", "StreamSums", "UnnormedRows",
            "build_part", "register_part", "registered",
-           "NormedDelta", "GatedAttention", "ParallelMixers", "Retention", "RecurrentGatedUnit", "ScaledPreNormBlock",
+           "NormedDelta", "GatedAttention", "DifferentialAttention", "GatedDeltaRule", "ParallelMixers", "Retention", "RecurrentGatedUnit", "ScaledPreNormBlock",
            "LatentAttention", "RoutedExperts", "SelectiveScan", "SandwichBlock", "NoFeedForward",
            "PairHashEmbedding", "Attention", "PreNormBlock", "Embedding", "LinearHead", "SwiGLU", "Linear", "RMSNorm", "NoPosition",
            "RotaryHalf"]

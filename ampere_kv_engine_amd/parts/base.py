@@ -242,13 +242,15 @@ class Unsettled:
 
 
 class ScaledDelta(Unsettled):
-    """A branch's output that is added to the residual sum times a constant: stream += scale * delta."""
+    """A branch's output that is added to the residual sum times a constant: stream += scale * delta - and then, where
+    the model's pass has given one, a vector `offset` that every row takes (what a pass over repeated layers adds before
+    its first layer).  `delta` None: the offset alone."""
 
-    def __init__(self, delta: torch.Tensor, scale: float, kernels):
-        self.delta, self.scale, self.kernels = delta, float(scale), kernels
+    def __init__(self, delta: torch.Tensor | None, scale: float, kernels, offset: torch.Tensor | None = None):
+        self.delta, self.scale, self.kernels, self.offset = delta, float(scale), kernels, offset
 
     def settle(self, stream: torch.Tensor) -> None:
-        self.kernels.norm_add_norm(stream, self.delta, None, 0.0, None, 0.0, None, delta_scale=self.scale)
+        self.kernels.norm_add_norm(stream, self.delta, None, 0.0, None, 0.0, None, delta_scale=self.scale, offset=self.offset)
 
 
 class NormedDelta(Unsettled):

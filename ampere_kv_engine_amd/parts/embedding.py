@@ -33,6 +33,49 @@ class Embedding(Part):
         return stream
 
 
+class NormedEmbedding(Embedding):
+    """The token's row, normed before the first layer: x = norm(table[id]), in float32 (one kernel).  `norm` is the
+    specification of an RMS norm whose weight is kept float32; its tensor is named `norm_name`."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        from .base import build_part
+        self.norm = build_part("norm", spec["norm"], runtime)
+        self.norm_name = spec["norm_name"]
+
+    def tensors(self, prefix=""):
+        return super().tensors() + self.norm.tensors(self.norm_name)
+
+    def load(self, fetch, prefix=""):
+        super().load(fetch)
+        self.norm.load(fetch, self.norm_name)
+
+    def forward(self, token_ids, stream, ctx=None):
+        self.rt.kernels.embed_normed(token_ids, self.weight, self.norm.weight, self.norm.eps, stream, ctx)
+        return stream
+
+
+class RowTable(Part):
+    """A table [rows, hidden] of vectors, float32, of which the model's pass adds one to every token's residual sum
+    where the run order says so (`RunEntry.adds_row`)."""
+    graph_safe = True
+
+    def __init__(self, spec, runtime):
+        self.rt = runtime
+        self.rows, self.hidden = int(spec["rows"]), int(spec["hidden_size"])
+        self.name = spec["name"]
+        self.table = None
+
+    def tensors(self, prefix=""):
+        return [TensorSpec(self.name, (self.rows, self.hidden), EMBEDDING)]
+
+    def load(self, fetch, prefix=""):
+        self.table = fetch(self.tensors()[0]).to(torch.float32).contiguous()
+
+    def row(self, index: int) -> torch.Tensor:
+        return self.table[index]
+
+
 class PairHashEmbedding(Embedding):
     """The token's row plus a row of a second table that is chosen by the token AND the one before it:
     row = (previous id * mul_prev + id * mul_cur) mod buckets; a request's first token takes the table's last row
@@ -91,4 +134,6 @@ class LinearHead(Part):
 
 register_part("embedding", "embedding", Embedding)
 register_part("embedding", "pair_hash_embedding", PairHashEmbedding)
+register_part("embedding", "normed_embedding", NormedEmbedding)
+register_part("embedding", "row_table", RowTable)
 register_part("head", "linear_head", LinearHead)

@@ -1,7 +1,8 @@
 """Feed-forwards.  `swiglu` is the dense gated one of the reference (ampere_kv/runner.py:172-177):
 down( silu(x Wg^T) * (x Wu^T) ), silu on the gate only.  Gate and up are one product: where the kernel set can, it
 also applies the activation before anything is stored (`gated_linear`); otherwise the stacked product is followed
-by the `swiglu` kernel."""
+by the `swiglu` kernel.  With `activation="gelu_tanh"` the gate passes the tanh form of gelu instead of silu: the stacked
+product, then the activation kernel that takes either (`gated_activation`)."""
 
 from __future__ import annotations
 
@@ -20,6 +21,9 @@ class SwiGLU(Part):
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
         self.name = spec.get("name", "mlp")
+        self.activation = spec.get("activation", "silu")
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"a gated feed-forward's activation is 'silu' or 'gelu_tanh', not {self.activation!r}")
         gate, up, down = spec.get("names", ("gate_proj.weight", "up_proj.weight", "down_proj.weight"))
         self.gate_up = Linear(runtime, self.hidden, [self.inter, self.inter], [gate, up])
         self.down = Linear(runtime, self.inter, [self.hidden], [down])
@@ -33,7 +37,8 @@ class SwiGLU(Part):
 
     def load(self, fetch, prefix):
         gate, up = (fetch(spec) for spec in self.gate_up.tensors(self._prefix(prefix)))
-        self.gated = self.rt.kernels.prepare_gated_linear(gate.contiguous(), up.contiguous())
+        self.gated = (self.rt.kernels.prepare_gated_linear(gate.contiguous(), up.contiguous())
+                      if self.activation == "silu" else None)        # (the one-pass product's epilogue is silu)
         if self.gated is None:
             self.gate_up.adopt(torch.cat((gate, up), dim=0).contiguous())
         else:
@@ -59,7 +64,10 @@ class SwiGLU(Part):
         else:
             gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
             self.gate_up.forward(x, gate_up)
-            self.rt.kernels.swiglu(gate_up, act)
+            if self.activation == "silu":
+                self.rt.kernels.swiglu(gate_up, act)
+            else:
+                self.rt.kernels.gated_activation(gate_up, act, self.activation)
         if ctx.fold_into_stream:     # the down product adds itself to the residual sum
             sums = self.down.add_to_stream(act, ctx)
             if sums is not None:

@@ -5,7 +5,10 @@
     a query at position i sees the keys j <= i - of its own chunk only, floor(i / chunk) = floor(j / chunk), where the
     mixer has chunks (counted from position 0 of the request); of the last `window` positions where it has a window
     weights: softmax - with `sink`, one more term exp(0) in the denominator that has no value:
-             p_j = exp(s_j) / (1 + sum exp(s_j))
+             p_j = exp(s_j) / (1 + sum exp(s_j)); with `sink="learned"` the term is exp(sink_h), a number per head (tensor
+             `sink`, kept float32)
+    with `position` (a `rope_scaled` specification): q and k are rotated over their first dims dimensions by the token's
+    position (after the unit norm, where there is one), inside the kernel that writes the keys to their pages
     head h's output times sigmoid(w_g[h] . h), one number per head and token (`head_gate`), before W_o.
 
 Keys are `head_dim` wide, values `value_dim`; query head h reads kv head h // (q_heads / kv_heads).  Keys are cached
@@ -14,7 +17,10 @@ after their norm.  All five projections are one product over the layer's input.
 
 from __future__ import annotations
 
-from .base import PagedKV, Part, SharesProducts, register_part
+import torch
+
+from ..weights.spec import BIAS, TensorSpec
+from .base import PagedKV, Part, SharesProducts, build_part, register_part
 from .linear import Linear
 
 
@@ -31,6 +37,11 @@ class GatedAttention(Part, SharesProducts):
         self.chunk = int(spec["chunk"]) if spec.get("chunk") is not None else None
         self.window = int(spec["window"]) if spec.get("window") is not None else None
         self.sink = bool(spec.get("sink", False))
+        self.learned_sink = spec.get("sink") == "learned"
+        self.sink_logits = None
+        self.position = build_part("position", spec["position"], runtime) if spec.get("position") is not None else None
+        if self.position is not None and self.position.dims > int(spec["head_dim"]):
+            raise ValueError(f"a rotation over {self.position.dims} dimensions does not fit heads of {spec['head_dim']}")
         self.unit_eps = float(spec["unit_norm_eps"]) if spec.get("unit_norm_eps") is not None else None
         self.head_gate = bool(spec.get("head_gate", False))
         self.name = spec.get("name", "attn")
@@ -42,8 +53,9 @@ class GatedAttention(Part, SharesProducts):
         if self.softcap is not None and self.softcap <= 0:
             raise ValueError(f"softcap must be positive or None, got {self.softcap}")
         self.q_size, self.k_size, self.v_size = self.q_heads * self.dim, self.kv_heads * self.dim, self.kv_heads * self.vdim
-        names = dict(q="q", k="k", v="v", g="g", o="o")
+        names = dict(q="q", k="k", v="v", g="g", o="o", sink="sink")
         names.update(spec.get("names") or {})
+        self.names = names
         bias = spec.get("bias_suffix")           # q, k and v have bias vectors named after them, with this suffix
         sizes, stacked = [self.q_size, self.k_size, self.v_size], [names["q"], names["k"], names["v"]]
         biases = [n + bias for n in stacked] if bias else None
@@ -54,20 +66,27 @@ class GatedAttention(Part, SharesProducts):
                 biases.append(None)
         self.width = sum(sizes)
         self.qkvg = self.inputs = Linear(runtime, self.hidden, sizes, stacked, bias_names=biases)
+        if self.learned_sink:
+            self.inputs = None      # (a tensor of its own beside the products: side by side with others it runs by itself)
         self.out = self.outputs = Linear(runtime, self.q_heads * self.vdim, [self.hidden], [names["o"]])
         runtime.kernels.check_gated_attention_sizes(self.q_heads, self.kv_heads, self.dim, self.vdim, runtime.page_size)
 
     def _prefix(self, prefix):
         return f"{prefix}{self.name}."
 
+    def _sink_spec(self, p):
+        return [TensorSpec(p + self.names["sink"], (self.q_heads,), BIAS)] if self.learned_sink else []
+
     def tensors(self, prefix):
         p = self._prefix(prefix)
-        return self.qkvg.tensors(p) + self.out.tensors(p)
+        return self.qkvg.tensors(p) + self.out.tensors(p) + self._sink_spec(p)
 
     def load(self, fetch, prefix):
         p = self._prefix(prefix)
         self.qkvg.load(fetch, p)
         self.out.load(fetch, p)
+        if self.learned_sink:
+            self.sink_logits = fetch(self._sink_spec(p)[0]).to(torch.float32).contiguous()
 
     def weight_bytes(self):
         return self.qkvg.weight_bytes() + self.out.weight_bytes()
@@ -80,12 +99,15 @@ class GatedAttention(Part, SharesProducts):
         k = self.rt.kernels
         meta = ctx.paged[cache.group]
         q = ctx.arena.take((projected.shape[0], self.q_size), self.rt.dtype)
+        rotation = {}
+        if self.position is not None:
+            rotation = dict(table=self.position.table, rot_dims=self.position.dims, positions=ctx.positions)
         k.unit_norm_write(projected, self.q_heads, self.kv_heads, self.dim, self.vdim, self.unit_eps,
-                          meta.slot_map if writes_cache else None, cache.k, cache.v, q, at=at)
+                          meta.slot_map if writes_cache else None, cache.k, cache.v, q, at=at, **rotation)
         k.gated_attention(q, cache.k, cache.v, projected if self.head_gate else None,
                           at + self.q_size + self.k_size + self.v_size, ctx, meta, self.q_heads, self.kv_heads, self.dim,
                           self.vdim, self.scale, self.softcap, self.chunk, self.window, self.sink, out, out_at=out_at,
-                          out_scale=out_scale)
+                          out_scale=out_scale, **({"sink_logits": self.sink_logits} if self.learned_sink else {}))
 
     def forward(self, x, ctx, cache, writes_cache: bool = True):
         tokens, dtype = x.shape[0], self.rt.dtype

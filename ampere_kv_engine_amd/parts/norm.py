@@ -5,14 +5,22 @@ file stores, so the product equals the reference's).
 With `single_rounding` the norm is float32 from the statistics to the product with the weight, and a result is
 rounded once, when it is stored (designs that say their norms are computed in 32-bit).  Such a norm takes no part in
 the folding of norms into products; it can be added to the residual sum as it is computed (`add_normed`) and chained
-with the norm that follows (`after`): the norm kernel of blocks that norm a branch before and after."""
+with the norm that follows (`after`): the norm kernel of blocks that norm a branch before and after.
+
+With `unit_offset` the file stores the weight around zero and the norm multiplies by 1 + w; the sum is formed once, at
+load, in float32."""
 
 from __future__ import annotations
 
 import torch
 
+from ..weights.random import NORM_STD, _normal, register_init_law
 from ..weights.spec import NORM, TensorSpec
 from .base import Norm, NormedDelta, ScaledDelta, StreamSums, UnnormedRows, register_part  # noqa: F401  (StreamSums is found here too)
+
+
+NORM_OFFSET = "norm_offset"          # a norm weight that is stored around zero and applied as 1 + w
+register_init_law(NORM_OFFSET, _normal(0.0, NORM_STD))
 
 
 class RMSNorm(Norm):
@@ -20,14 +28,21 @@ class RMSNorm(Norm):
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
         self.single_rounding = bool(spec.get("single_rounding", False))
+        self.unit_offset = bool(spec.get("unit_offset", False))
         self.rt = runtime
         self.weight: torch.Tensor | None = None
 
+    @property
+    def role(self) -> str:
+        return NORM_OFFSET if self.unit_offset else NORM
+
     def tensors(self, name: str):
-        return [TensorSpec(name, (self.size,), NORM)]
+        return [TensorSpec(name, (self.size,), self.role)]
 
     def load(self, fetch, name: str):
-        self.weight = fetch(TensorSpec(name, (self.size,), NORM)).to(torch.float32).contiguous()
+        self.weight = fetch(TensorSpec(name, (self.size,), self.role)).to(torch.float32).contiguous()
+        if self.unit_offset:
+            self.weight += 1.0
 
     def weight_bytes(self):
         return self.size * 4
@@ -58,7 +73,9 @@ class RMSNorm(Norm):
 
     def after(self, stream, pending, out):
         if isinstance(pending, ScaledDelta) and self.single_rounding:      # one kernel: add the branch times its constant, norm
-            return self.forward_residual(stream, pending.delta, out, delta_scale=pending.scale)
+            self.rt.kernels.norm_add_norm(stream, pending.delta, None, 0.0, self.weight, self.eps, out,
+                                          delta_scale=pending.scale, offset=pending.offset)
+            return out
         if (pending is None or not isinstance(pending, NormedDelta)
                 or not (self.single_rounding and type(pending.norm) is RMSNorm and pending.norm.single_rounding)):
             return super().after(stream, pending, out)

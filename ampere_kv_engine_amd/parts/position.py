@@ -1,6 +1,16 @@
 """Position encodings.  `rope_half` is the rotary encoding with pairs (j, j + d/2) over the whole head
 (ampere_kv/runner.py:80-98): angle = position * theta^(-2j/d) in float32; x' = x cos + rot(x) sin with
-rot(x) = cat(-x[d/2:], x[:d/2]).  `none` leaves q and k as they are."""
+rot(x) = cat(-x[d/2:], x[:d/2]).  `none` leaves q and k as they are.
+
+`rope_scaled` is a table for mixers that rotate the first `dims` dimensions of a head themselves, with frequencies
+f_i = base^(-2i / dims) that a rule stretches for contexts longer than the `original` one:
+  * "yarn": with dim(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(dim(fast)), 0), hi =
+    min(ceil(dim(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1):
+    f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i); cos and sin are multiplied by 0.1 ln(factor) + 1;
+  * "llama3": with the wavelength l_i = 2 pi / f_i: f_i stays where l_i < original / high, becomes f_i / factor where
+    l_i > original / low, and between the two, with s = (original / l_i - low) / (high - low), (1 - s) f_i / factor + s f_i;
+  * none: the frequencies as they are.
+Frequencies are formed in double precision and rounded once; angles are float32 products of position and frequency."""
 
 from __future__ import annotations
 
@@ -32,6 +42,66 @@ class RotaryHalf(Part):
         return x
 
 
+def stretched_frequencies(dims: int, base: float, scaling) -> tuple[list[float], float]:
+    """(the dims / 2 frequencies, the factor on cos and sin) under `scaling`: None, or a mapping with `kind` ("yarn":
+    factor, original, fast, slow; "llama3": factor, original, low, high)."""
+    import math
+    freqs = [base ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if scaling is None:
+        return freqs, 1.0
+    kind, factor, original = scaling["kind"], float(scaling["factor"]), float(scaling["original"])
+    if kind == "yarn":
+        turned = lambda turns: dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+        lo = max(math.floor(turned(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turned(float(scaling["slow"]))), dims - 1)
+        out = []
+        for i, f in enumerate(freqs):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(f / factor * ramp + f * (1.0 - ramp))
+        return out, 0.1 * math.log(factor) + 1.0
+    if kind == "llama3":
+        low, high = float(scaling["low"]), float(scaling["high"])
+        out = []
+        for f in freqs:
+            wavelength = 2.0 * math.pi / f
+            if wavelength < original / high:
+                out.append(f)
+            elif wavelength > original / low:
+                out.append(f / factor)
+            else:
+                share = (original / wavelength - low) / (high - low)
+                out.append((1.0 - share) * f / factor + share * f)
+        return out, 1.0
+    raise ValueError(f"frequencies are stretched by 'yarn' or 'llama3', not {kind!r}")
+
+
+class ScaledRotary(Part):
+    """The cos/sin table of a rotation over a head's first `dims` dimensions with stretched frequencies; the mixer that
+    owns it rotates inside its own kernels (`table`, `dims`).  One table for all layers with the same constants."""
+
+    def __init__(self, spec, runtime):
+        self.rt = runtime
+        self.dims, self.base = int(spec["dims"]), float(spec["base"])
+        scaling = spec.get("scaling")
+        if self.dims <= 0 or self.dims % 2:
+            raise ValueError(f"a rotation turns an even number of dimensions, got {self.dims}")
+        freqs, magnitude = stretched_frequencies(self.dims, self.base, scaling)
+        self.magnitude = magnitude
+        half = self.dims // 2
+        reach = (runtime.max_seq_len + runtime.page_size - 1) // runtime.page_size * runtime.page_size     # whole pages
+        key = ("rope_scaled", self.dims, self.base, tuple(sorted(scaling.items())) if scaling is not None else None, reach)
+        freq = torch.tensor(freqs, dtype=torch.float64).to(torch.float32)
+
+        def fill(table):
+            runtime.kernels.rope_table(freq.to(runtime.device), table)
+            if magnitude != 1.0:
+                table.mul_(magnitude)
+        self.table = runtime.shared_buffer(key, (reach, half, 2), torch.float32, fill)
+
+    def apply(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError("a stretched rotation is applied by the mixer that owns it, inside its kernels")
+
+
 class NoPosition(Part):
     def __init__(self, spec, runtime):
         self.table = None
@@ -42,3 +112,4 @@ class NoPosition(Part):
 
 register_part("position", "rope_half", RotaryHalf)
 register_part("position", "none", NoPosition)
+register_part("position", "rope_scaled", ScaledRotary)

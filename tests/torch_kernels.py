@@ -267,14 +267,68 @@ class TorchKernels(KernelSet):
         out.copy_(table[cur].float() + pairs[rows].float())
         words[ctx.seq_slots.long(), 7] = cur[ctx.q_start.long()[1:] - 1].int()
 
-    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale=1.0):
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale=1.0, offset=None):
         if delta is not None:
             d = delta.float() * delta_scale
             if post_weight is not None:
                 d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight
             stream += d
+        if offset is not None:
+            stream += offset
         if out is not None:
             out.copy_((stream * torch.rsqrt((stream * stream).mean(-1, keepdim=True) + pre_eps) * pre_weight).to(out.dtype))
+
+    def embed_normed(self, ids, table, weight, eps, out, ctx=None):
+        """out[n] = table[id] / rms(table[id]) * weight; an id of -1 is the token chosen last for the row's request."""
+        self.embed(ids, table, out, ctx)
+        out.copy_(out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps) * weight)
+
+    def gated_activation(self, gate_up, out, activation):
+        inter = out.shape[1]
+        gate, up = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+        if activation == "gelu_tanh":
+            act = 0.5 * gate * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (gate + 0.044715 * gate ** 3)))
+        else:
+            act = gate * torch.sigmoid(gate)
+        out.copy_((act * up).to(out.dtype))
+
+    def difference_norm_gate(self, maps, lam, eps, after, gates, gate_at, heads, vdim, out):
+        n = maps.shape[0]
+        both = maps.float().view(n, heads, 2, vdim)
+        o = both[:, :, 0] - lam.float() * both[:, :, 1]
+        o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * after
+        gate = torch.sigmoid(gates[:, gate_at:gate_at + heads * vdim].float()).view(n, heads, vdim)
+        out.copy_((o * gate).reshape(n, heads * vdim).to(out.dtype))
+
+    def check_delta_rule_sizes(self, heads, groups, dim, vdim):
+        assert heads % groups == 0
+
+    def delta_rule(self, conv, beta_logits, beta_at, decay_logits, decay_bias, rate, gates, norm_weight, unit_eps, norm_eps,
+                   q_scale, heads, groups, dim, vdim, state, ctx, out):
+        """S of a request lies at the start of its slot as [heads, vdim, dim]."""
+        n = conv.shape[0]
+        x = conv.float()
+        qk = groups * dim
+        q, k = x[:, :qk].reshape(n, groups, dim), x[:, qk:2 * qk].reshape(n, groups, dim)
+        v = x[:, 2 * qk:].reshape(n, heads, vdim)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * q_scale
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+        share = heads // groups
+        q, k = q.repeat_interleave(share, dim=1), k.repeat_interleave(share, dim=1)
+        beta = torch.sigmoid(beta_logits[:, beta_at:beta_at + heads].float())
+        g = torch.exp(-rate[None, :, None] * torch.nn.functional.softplus(
+            (decay_logits + decay_bias).view(n, heads, dim), threshold=20.0))
+        for r in range(ctx.num_seqs):
+            first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
+            S = state[slot, :heads * dim * vdim].view(heads, vdim, dim).transpose(1, 2).clone()      # [heads, dim, vdim]
+            for t in range(first, last):
+                S = g[t][:, :, None] * S
+                u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+                S = S + k[t][:, :, None] * u[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, q[t])
+                o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + norm_eps) * norm_weight
+                out[t] = (o * torch.sigmoid(gates[t].view(heads, vdim))).reshape(-1).to(out.dtype)
+            state[slot, :heads * dim * vdim] = S.transpose(1, 2).reshape(-1)
 
     @staticmethod
     def _turn(x, positions, table, rot_dims):
@@ -324,17 +378,19 @@ class TorchKernels(KernelSet):
                 weights = ((q_abs[n] @ recs.T) * scale).softmax(-1)             # [heads, S]
                 out[n] = weights @ recs[:, :kv_rank]
 
-    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation="silu"):
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation="silu", conv_at=None):
         taps = weight.shape[1]
-        conv_at = channels * n_state
+        if conv_at is None:
+            conv_at = channels * n_state
+        conv_end = conv_at + (taps - 1) * channels
         for r in range(ctx.num_seqs):
             first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
-            kept = state[slot, conv_at:].view(taps - 1, channels)
+            kept = state[slot, conv_at:conv_end].view(taps - 1, channels)
             seen = torch.cat((kept, xz[first:last, :channels].float()), dim=0)
             for t in range(last - first):
-                acc = (seen[t:t + taps] * weight.float().T).sum(0) + bias.float()
+                acc = (seen[t:t + taps] * weight.float().T).sum(0) + (bias.float() if bias is not None else 0.0)
                 out[first + t] = (acc * torch.sigmoid(acc) if activation == "silu" else acc).to(out.dtype)
-            state[slot, conv_at:] = seen[seen.shape[0] - (taps - 1):].reshape(-1)
+            state[slot, conv_at:conv_end] = seen[seen.shape[0] - (taps - 1):].reshape(-1)
 
     def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out):
         channels, n_state = a.shape
@@ -374,26 +430,32 @@ class TorchKernels(KernelSet):
     def check_retention_sizes(self, heads, dim, vdim):
         pass
 
-    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at=0):
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at=0, maps=1,
+                        table=None, rot_dims=0, positions=None):
         projected = projected[:, at:]
         n = projected.shape[0]
-        q_size, k_size, v_size = q_heads * dim, kv_heads * dim, kv_heads * vdim
-        q = projected[:, :q_size].reshape(n, q_heads, dim).float()
-        k = projected[:, q_size:q_size + k_size].reshape(n, kv_heads, dim).float()
+        q_size, k_size, v_size = q_heads * maps * dim, kv_heads * maps * dim, kv_heads * vdim
+        q = projected[:, :q_size].reshape(n, q_heads * maps, dim).float()
+        k = projected[:, q_size:q_size + k_size].reshape(n, kv_heads * maps, dim).float()
         v = projected[:, q_size + k_size:q_size + k_size + v_size].reshape(n, kv_heads, vdim)
         if eps is not None:
             q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)
             k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)
+        if table is not None:
+            q, k = self._turn(q, positions, table, rot_dims), self._turn(k, positions, table, rot_dims)
         q_out.copy_(q.reshape(n, q_size).to(q_out.dtype))
         if slot_map is not None:
             page_size = k_pages.shape[2]
             slots = slot_map.long()
-            k_pages[slots // page_size, :, slots % page_size] = k.to(k_pages.dtype)
+            k_pages[slots // page_size, :, slots % page_size] = k.reshape(n, kv_heads, maps * dim).to(k_pages.dtype)
             v_pages[slots // page_size, :, :, slots % page_size] = v.to(v_pages.dtype)
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
-                        chunk, window, sink, out, out_at=0, out_scale=1.0):
+                        chunk, window, sink, out, out_at=0, out_scale=1.0, sink_logits=None, maps=1):
+        """`maps` > 1: a head has `maps` query vectors; vector number m of a head reads the m-th `dim` columns of its key
+        head's record and the head's values.  `sink_logits`: the sink's term is exp(sink_logits[head])."""
         page_size = k_pages.shape[2]
+        q_heads = q_heads * maps          # (from here on: query vectors)
         group = q_heads // kv_heads
         table = meta.block_table.cpu()
         if getattr(meta, "rows", None) is not None:
@@ -421,15 +483,17 @@ class TorchKernels(KernelSet):
                 visible &= (key_pos[None, :] // chunk) == (q_pos[:, None] // chunk)
             merged = torch.empty(last - first, q_heads, vdim)
             for head in range(q_heads):
-                scores = (qs[:, head] @ keys[:, head // group].T) * scale
+                record = keys[:, head // group]
+                scores = (qs[:, head] @ record[:, head % maps * dim:head % maps * dim + dim].T) * scale
                 if softcap is not None:
                     scores = softcap * torch.tanh(scores / softcap)
                 scores = scores.masked_fill(~visible, -math.inf)
                 top = scores.amax(-1, keepdim=True)
+                sunk = float(sink_logits[head]) if sink_logits is not None else 0.0
                 if sink:
-                    top = top.clamp(min=0.0)
+                    top = top.clamp(min=sunk)
                 weights = torch.exp(scores - top)
-                total = weights.sum(-1, keepdim=True) + (torch.exp(-top) if sink else 0.0)
+                total = weights.sum(-1, keepdim=True) + (torch.exp(sunk - top) if sink else 0.0)
                 merged[:, head] = (weights / total) @ values[:, head // group]
             if gates is not None:
                 merged = merged * torch.sigmoid(gates[first:last, gate_at:gate_at + q_heads].float())[:, :, None]
