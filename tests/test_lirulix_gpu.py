@@ -62,7 +62,9 @@ def test_one_mechanism_alone(mechanism, dtype, tmp_path):
 
 def test_steps_are_recorded_and_replayed(case):
     """Decode steps come again and again: the second is recorded, the later ones are replays; all agree with the plain
-    implementation, and an engine that records nothing gives the same bits."""
+    implementation, and with an engine that records nothing to a few units in the last place (a recording cuts a row's keys
+    over waves by a bound on the request's length, an eager step by the length itself: the order of the sums differs where
+    no window bounds the keys)."""
     ids = case["requests"]["d"]
     want = case["expected"]["d"]
     outs = {}
@@ -73,7 +75,7 @@ def test_steps_are_recorded_and_replayed(case):
         outs[graphs] = got["d"]
         if graphs:
             assert any(g is not None for g in engine._graphs.values()), "nothing was recorded"
-    assert torch.equal(outs[True], outs[False])
+    torch.testing.assert_close(outs[True], outs[False], rtol=0, atol=2e-5 * float(want.abs().max()))
 
 
 def test_trace_replay_of_a_random_model(case, tmp_path):
