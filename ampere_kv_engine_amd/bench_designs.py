@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the Keranex design (and, `--workload tukevik`, of the Tukevik design) at sizes that resemble a real model's layers (random weights),
+"""Prefill and decode throughput of the Keranex design (and, `--workload tukevik` / `lirulix`, of those designs) at sizes that resemble a real model's layers (random weights),
 beside the dense Qwen3 decoder at equal width, depth, heads and active feed-forward width - the closest model the
 engine has.  `python bench.py --workload keranex [--design-sizes s,m] [--layers L]` prints one JSON line per size:
 
@@ -71,6 +71,48 @@ def tukevik_config(size: dict, layers: int) -> dict:
                 layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer, mlp in (pattern[i % 4] for i in range(layers))])
 
 
+# Lirulix at the same widths: the pattern [attention with a sink, delta rule, attention with a sink, differential
+# attention over a window], every layer with a dense feed-forward, all layers inside one pass of the loop.  Beside it
+# Tukevik (the closest design the engine has: attention with a sink on the same kernels, a mixer with a matrix state per
+# head, float32 norms) with the same width, depth, heads and feed-forward width, its feed-forwards all dense.
+LIRULIX_SIZES = {
+    "s": dict(width=2048, vocab=32768, heads=16, kv_heads=4, dim=128, vdim=128, rot=64, d_heads=16, d_kv_heads=4, d_dim=64,
+              d_vdim=128, window=1024, r_heads=16, r_kv_heads=16, r_dim=128, r_vdim=128, conv=4, decay_rank=64, gate_rank=64,
+              ff=3072),
+    "m": dict(width=4096, vocab=65536, heads=32, kv_heads=8, dim=128, vdim=128, rot=64, d_heads=32, d_kv_heads=8, d_dim=64,
+              d_vdim=128, window=2048, r_heads=32, r_kv_heads=32, r_dim=128, r_vdim=128, conv=4, decay_rank=128, gate_rank=128,
+              ff=5120),
+}
+
+
+def lirulix_config(size: dict, layers: int) -> dict:
+    sink = dict(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], vdim=size["vdim"], scale=size["dim"] ** -0.5,
+                rot=dict(dims=size["rot"], base=1e6, scaling=dict(factor=4.0, original=4096, fast=32.0, slow=1.0)))
+    two = dict(heads=size["d_heads"], kv_heads=size["d_kv_heads"], dim=size["d_dim"], vdim=size["d_vdim"], diff=0.3,
+               scale=size["d_dim"] ** -0.5, mask=dict(size=size["window"]),
+               rot=dict(dims=size["d_dim"], base=1e4, scaling=dict(factor=8.0, original=8192, low=1.0, high=4.0)))
+    delta = dict(heads=size["r_heads"], kv_heads=size["r_kv_heads"], dim=size["r_dim"], vdim=size["r_vdim"], conv=size["conv"],
+                 ranks=dict(decay=size["decay_rank"], gate=size["gate_rank"]))
+    mlp = dict(kind="dense", ff=size["ff"])
+    pattern = [("attention", sink), ("channel_delta", delta), ("attention", sink), ("attention_2", two)]
+    return dict(architecture="Lirulix", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6),
+                layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer in (pattern[i % 4] for i in range(layers))],
+                loop=dict(start=0, stop=layers, times=1))
+
+
+def tukevik_beside_lirulix(size: dict, layers: int) -> dict:
+    parallel = dict(
+        left=dict(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], vdim=size["vdim"], mask=dict(size=4096),
+                  scale=size["dim"] ** -0.5, softcap=50.0), left_scale=0.7,
+        right=dict(heads=size["r_heads"] // 4, dim=size["r_dim"], vdim=size["r_vdim"], rot=dict(base=1e4, dims=size["r_dim"]),
+                   decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(size["r_heads"] // 4)]), right_scale=1.2)
+    recurrent = dict(width=size["width"], blocks=16, conv=size["conv"])
+    mlp = dict(kind="dense", ff=size["ff"])
+    pattern = [("parallel", parallel), ("rglru", recurrent)]
+    return dict(architecture="Tukevik", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6), residual_mult=0.6,
+                layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer in (pattern[i % 2] for i in range(layers))])
+
+
 def qwen3_beside_tukevik(size: dict, layers: int) -> dict:
     return dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers, hidden_size=size["width"],
                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
@@ -137,7 +179,22 @@ def measure(config, batch: int, context: int, steps: int, warmup: int, graphs: b
 
 def design_workload(sizes: str, layers: int | None, batch: int, context: int, steps: int, warmup: int,
                     graphs: bool = True, only: str = "", design: str = "keranex") -> int:
-    from .config import KeranexConfig, Qwen3Config, TukevikConfig
+    from .config import KeranexConfig, LirulixConfig, Qwen3Config, TukevikConfig
+    for name in [s for s in sizes.split(",") if s and design == "lirulix"]:
+        size = LIRULIX_SIZES[name]
+        count = layers or 8
+        line = {"workload": "lirulix", "sizes": name, "layers": count, "batch": batch, "context": context,
+                "prefill_tokens": PREFILL_TOKENS, "dtype": "bf16", "data": "synthetic: random-init weights, random token ids",
+                "shape": size}
+        if only in ("", "lirulix"):
+            line["lirulix"] = measure(LirulixConfig.from_dict(lirulix_config(size, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "tukevik"):
+            line["tukevik_equal_size"] = measure(TukevikConfig.from_dict(tukevik_beside_lirulix(size, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "qwen3"):
+            line["qwen3_equal_size"] = measure(Qwen3Config.from_dict(qwen3_beside_tukevik(dict(size, dense=size["ff"]), count)), batch, context, steps, warmup, graphs)
+        print(json.dumps(line), flush=True)
+    if design == "lirulix":
+        return 0
     for name in [s for s in sizes.split(",") if s and design == "tukevik"]:
         size = TUKEVIK_SIZES[name]
         count = layers or 8

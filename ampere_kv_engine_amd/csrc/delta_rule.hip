@@ -6,12 +6,14 @@
 //
 // Three kernels.  `delta_prepare` is token-wise: the unit vectors, decays, betas and k . q of every token, float32, into a
 // workspace.  `delta_recur` walks a request's tokens: a column of S is spread over R neighbouring lanes (RP rows each), so
-// S^T k and S^T q are sums over RP registers and a butterfly over R lanes, and columns need nothing of each other - a
-// block takes 256 / R columns of one head, the device as many blocks as heads x columns allow.  Since
-// (g S + k u^T)^T q = (g S)^T q + u (k . q), both sums are taken over the decayed state in one pass.  A tile of tokens'
-// q, k and g passes through LDS for all columns of the block.  `delta_finish` is token-wise again: o / rms(o) times a
-// weight per value channel and the sigmoid of a gate.  A request's state lies in its slot transposed, [heads, vdim, dim]:
-// a lane's rows of a column are consecutive floats.
+// S^T k and S^T q are sums over RP registers and a butterfly over R lanes inside the vector unit, and columns need nothing
+// of each other - a block takes 256 / R columns of one head.  The recurrence is a chain through the tokens whose length
+// nothing shortens, so what counts is a wave's instructions per token: with four rows a lane, one request's heads of
+// 128 x 128 are 1,024 waves - one on every vector unit of the device.  Since (g S + k u^T)^T q = (g S)^T q + u (k . q),
+// both sums are taken over the decayed state in one pass.  A tile of tokens' q, k and g passes through LDS for all columns
+// of the block; the next tile's values are asked for before this tile's tokens are walked.  `delta_finish` is token-wise
+// again: o / rms(o) times a weight per value channel and the sigmoid of a gate.  A request's state lies in its slot
+// transposed, [heads, vdim, dim]: a lane's rows of a column are consecutive floats.
 
 #include "common.h"
 #include "api_parts.h"
@@ -28,8 +30,10 @@ __host__ __device__ inline long prepared_width(int heads, int groups, int dim) {
   return 2L * groups * dim + static_cast<long>(heads) * dim + 2L * heads;
 }
 
-// One block per token.  conv rows: [q (groups x dim) | k (groups x dim) | v ...] after convolution and activation;
-// beta_logits at `beta_stride` per token; decay_logits [tokens, heads x dim] float32.
+// A wave is a token's unit of work: units 0 .. groups - 1 are a q / k pair (sums of squares and the product from one pass
+// over the raw vectors: k . q of the unit vectors follows without reading them back; the betas of the pair's heads go
+// along), every further unit 256 decays.  conv rows: [q (groups x dim) | k (groups x dim) | v ...] after convolution and
+// activation; beta_logits at `beta_stride` per token; decay_logits [tokens, heads x dim] float32.
 template <typename T>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict__ conv, long conv_stride,
                                                             const T* __restrict__ beta_logits, long beta_stride,
@@ -38,95 +42,171 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const T* __restrict_
                                                             const float* __restrict__ rate, float unit_eps, float q_scale,
                                                             float* __restrict__ prepared, int heads, int groups, int dim) {
   const long n = blockIdx.x;
-  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int unit = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
   const long width = prepared_width(heads, groups, dim);
   float* row = prepared + n * width;
-  const T* x = conv + n * conv_stride;
-  // unit vectors: a wave a vector (queries first, then keys)
-  for (int item = wave; item < 2 * groups; item += waves) {
-    const T* src = x + static_cast<long>(item) * dim;
-    float squares = 0.f;
-    for (int i = lane; i < dim; i += kWave) {
-      const float v = to_float(src[i]);
-      squares += v * v;
-    }
-    const float scale = (item < groups ? q_scale : 1.f) / sqrtf(wave_sum(squares) + unit_eps);
-    for (int i = lane; i < dim; i += kWave) row[static_cast<long>(item) * dim + i] = to_float(src[i]) * scale;
-  }
   float* g = row + 2L * groups * dim;
-  for (int i = threadIdx.x; i < heads * dim; i += blockDim.x)
-    g[i] = expf(-rate[i / dim] * softplus_of(decay_logits[n * heads * dim + i] + decay_bias[i]));
   float* beta = g + static_cast<long>(heads) * dim;
-  for (int h = threadIdx.x; h < heads; h += blockDim.x) beta[h] = sigmoid_of(to_float(beta_logits[n * beta_stride + h]));
-  __syncthreads();       // the unit vectors of this token are in memory: k . q per head, a wave a head
   const int share = heads / groups;
-  for (int h = wave; h < heads; h += waves) {
-    const float* qs = row + static_cast<long>(h / share) * dim;
-    const float* ks = row + static_cast<long>(groups + h / share) * dim;
-    float dot = 0.f;
-    for (int i = lane; i < dim; i += kWave) dot = fmaf(qs[i], ks[i], dot);
-    dot = wave_sum(dot);
-    if (lane == 0) beta[heads + h] = dot;
+  if (unit < groups) {
+    const T* qs = conv + n * conv_stride + static_cast<long>(unit) * dim;
+    const T* ks = qs + static_cast<long>(groups) * dim;
+    float qq = 0.f, kk = 0.f, qk = 0.f;
+    for (int i = lane; i < dim; i += kWave) {
+      const float a = to_float(qs[i]), b = to_float(ks[i]);
+      qq = fmaf(a, a, qq), kk = fmaf(b, b, kk), qk = fmaf(a, b, qk);
+    }
+    const float q_unit = q_scale / sqrtf(wave_sum(qq) + unit_eps), k_unit = 1.f / sqrtf(wave_sum(kk) + unit_eps);
+    const float dot = wave_sum(qk) * q_unit * k_unit;
+    for (int i = lane; i < dim; i += kWave) {
+      row[static_cast<long>(unit) * dim + i] = to_float(qs[i]) * q_unit;
+      row[static_cast<long>(groups + unit) * dim + i] = to_float(ks[i]) * k_unit;
+    }
+    for (int j = lane; j < share; j += kWave) {
+      const int h = unit * share + j;
+      beta[h] = sigmoid_of(to_float(beta_logits[n * beta_stride + h]));
+      beta[heads + h] = dot;
+    }
+    return;
+  }
+  const int first = (unit - groups) * 256;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int i = first + e * kWave + lane;
+    if (i < heads * dim) g[i] = expf(-rate[i / dim] * softplus_of(decay_logits[n * heads * dim + i] + decay_bias[i]));
   }
 }
 
+// Sums over the R neighbouring lanes of a column, in all of them, without a trip through LDS: exchanges inside quads, the
+// two mirrors of a row of 16 lanes, then swaps of rows and of the wave's halves.
+template <int CTRL> __device__ __forceinline__ float lane_exchange(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int R> __device__ __forceinline__ float column_sum(float v) {
+  if (R >= 2) v += lane_exchange<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+  if (R >= 4) v += lane_exchange<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+  if (R >= 8) v += lane_exchange<0x141>(v);      // row_half_mirror
+  if (R >= 16) v += lane_exchange<0x140>(v);     // row_mirror
+  if (R >= 32) {
+    const uint32_t bits = __float_as_uint(v);
+    const auto swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    v = __uint_as_float(swapped[0]) + __uint_as_float(swapped[1]);
+  }
+  if (R >= 64) {
+    const uint32_t bits = __float_as_uint(v);
+    const auto swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    v = __uint_as_float(swapped[0]) + __uint_as_float(swapped[1]);
+  }
+  return v;
+}
+
+// Tokens of a tile: what 48 KB of LDS hold of their q, k and g, 16 at most.
+template <int RP, int R> struct DeltaTile {
+  static constexpr int kSegment = RP == 4 ? 4 : RP + 4;     // (padding keeps the longer segments of neighbouring lanes in different banks)
+  static constexpr int kArray = R * kSegment;
+  static constexpr int kColumns = 256 / R;
+  static constexpr int kTokens = (12288 / (3 * kArray)) >= 16 ? 16 : (12288 / (3 * kArray)) >= 1 ? (12288 / (3 * kArray)) : 1;
+  static constexpr int kFloats = kTokens * (3 * kArray + kColumns + 2);
+};
+
 // A block: one request, one head, 256 / R columns of S.  Thread (column, part): rows part * RP .. part * RP + RP - 1.
-// LDS: per token of a tile three arrays (q, k, g) of R segments of RP + 4 floats (the padding keeps the segments of
-// neighbouring lanes in different banks), then the tile's values [tile][columns] and betas and k . q [tile][2].
-template <typename T, int RP>
+// LDS: per token of a tile three arrays (q, k, g) of R segments, then the tile's values [tile][columns] and its betas and
+// k . q [tile][2].
+template <typename T, int RP, int R>
 __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restrict__ prepared, const T* __restrict__ conv,
                                                           long conv_stride, long v_at, float* __restrict__ state,
                                                           long state_stride, const int* __restrict__ q_start,
                                                           const int* __restrict__ seq_slots, float* __restrict__ raw_out,
-                                                          int heads, int groups, int dim, int vdim, int R, int tile) {
-  extern __shared__ float lds[];
-  constexpr int SP = RP + 4;
-  const int columns = 256 / R, column_blocks = (vdim + columns - 1) / columns;
+                                                          int heads, int groups, int dim, int vdim) {
+  using Tile = DeltaTile<RP, R>;
+  constexpr int SP = Tile::kSegment, kArray = Tile::kArray, kColumns = Tile::kColumns, kTile = Tile::kTokens;
+  constexpr int kPadded = R * RP;
+  constexpr int kVectorLoads = (kTile * kPadded + 255) / 256, kValueLoads = (kTile * kColumns + 255) / 256;
+  __shared__ float lds[Tile::kFloats];
+  float* values = lds + kTile * 3 * kArray;        // [tile][columns]
+  float* scalars = values + kTile * kColumns;      // [tile][2]: beta, k . q
+  const int column_blocks = (vdim + kColumns - 1) / kColumns;
   const int r = blockIdx.x / (heads * column_blocks);
   const int h = blockIdx.x / column_blocks % heads;
   const int part = threadIdx.x % R;
-  const int col = blockIdx.x % column_blocks * columns + threadIdx.x / R;
+  const int col0 = blockIdx.x % column_blocks * kColumns;
+  const int col = col0 + threadIdx.x / R;
   const bool works = col < vdim;
   const int first = q_start[r], last = q_start[r + 1];
   const long width = prepared_width(heads, groups, dim);
   const int share = heads / groups;
   const long q_off = static_cast<long>(h / share) * dim, k_off = static_cast<long>(groups + h / share) * dim;
   const long g_off = 2L * groups * dim + static_cast<long>(h) * dim, b_off = 2L * groups * dim + static_cast<long>(heads) * dim + h;
-  const int array = R * SP, token_floats = 3 * array;
-  float* values = lds + static_cast<long>(tile) * token_floats;       // [tile][columns]
-  float* scalars = values + static_cast<long>(tile) * columns;        // [tile][2]: beta, k . q
 
   float S[RP];
   float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + (static_cast<long>(h) * vdim + (works ? col : 0)) * dim;
+  const bool whole_fours = dim % 4 == 0 && state_stride % 4 == 0;      // (16-byte accesses need their alignment)
 #pragma unroll
-  for (int i = 0; i < RP; ++i) {
+  for (int i = 0; i < RP; i += 4) {
     const int d = part * RP + i;
-    S[i] = works && d < dim ? kept[d] : 0.f;
+    if (works && whole_fours && d < dim) {
+      const float4 four = *reinterpret_cast<const float4*>(kept + d);
+      S[i] = four.x, S[i + 1] = four.y, S[i + 2] = four.z, S[i + 3] = four.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) S[i + e] = works && d + e < dim ? kept[d + e] : 0.f;
+    }
   }
-  const int padded = R * RP;
-  for (int t0 = first; t0 < last; t0 += tile) {
-    const int count = min(tile, last - t0);
-    __syncthreads();          // the tile before has been used by everybody
-    for (int index = threadIdx.x; index < count * padded; index += blockDim.x) {
-      const int tt = index / padded, d = index % padded;
+
+  // a tile's operands on their way from memory: asked for one tile ahead, laid into LDS when the tile before is done
+  float fetched_q[kVectorLoads], fetched_k[kVectorLoads], fetched_g[kVectorLoads], fetched_v[kValueLoads], fetched_s = 0.f;
+  auto fetch = [&](int t0) {
+    const int count = min(kTile, last - t0);
+#pragma unroll
+    for (int j = 0; j < kVectorLoads; ++j) {
+      const int index = threadIdx.x + j * 256;
+      const int tt = index / kPadded, d = index % kPadded;
+      const bool real = tt < count && d < dim;
       const float* row = prepared + static_cast<long>(t0 + tt) * width;
-      float* at = lds + static_cast<long>(tt) * token_floats + (d / RP) * SP + d % RP;
-      const bool real = d < dim;
-      at[0] = real ? row[q_off + d] : 0.f;
-      at[array] = real ? row[k_off + d] : 0.f;
-      at[2 * array] = real ? row[g_off + d] : 1.f;
+      fetched_q[j] = real ? row[q_off + d] : 0.f;
+      fetched_k[j] = real ? row[k_off + d] : 0.f;
+      fetched_g[j] = real ? row[g_off + d] : 1.f;
     }
-    for (int index = threadIdx.x; index < count * columns; index += blockDim.x) {
-      const int tt = index / columns, c = blockIdx.x % column_blocks * columns + index % columns;
-      values[index] = c < vdim ? to_float(conv[static_cast<long>(t0 + tt) * conv_stride + v_at + static_cast<long>(h) * vdim + c]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < kValueLoads; ++j) {
+      const int index = threadIdx.x + j * 256;
+      const int tt = index / kColumns, c = col0 + index % kColumns;
+      fetched_v[j] = tt < count && c < vdim
+                         ? to_float(conv[static_cast<long>(t0 + tt) * conv_stride + v_at + static_cast<long>(h) * vdim + c]) : 0.f;
     }
-    for (int index = threadIdx.x; index < count * 2; index += blockDim.x)
-      scalars[index] = prepared[static_cast<long>(t0 + index / 2) * width + b_off + (index & 1) * heads];
+    const int which = threadIdx.x;
+    fetched_s = which < 2 * count ? prepared[static_cast<long>(t0 + which / 2) * width + b_off + (which & 1) * heads] : 0.f;
+  };
+  auto lay_down = [&]() {
+#pragma unroll
+    for (int j = 0; j < kVectorLoads; ++j) {
+      const int index = threadIdx.x + j * 256;
+      if (index >= kTile * kPadded) continue;
+      const int tt = index / kPadded, d = index % kPadded;
+      float* at = lds + tt * 3 * kArray + (d / RP) * SP + d % RP;
+      at[0] = fetched_q[j], at[kArray] = fetched_k[j], at[2 * kArray] = fetched_g[j];
+    }
+#pragma unroll
+    for (int j = 0; j < kValueLoads; ++j) {
+      const int index = threadIdx.x + j * 256;
+      if (index < kTile * kColumns) values[index] = fetched_v[j];
+    }
+    if (threadIdx.x < 2 * kTile) scalars[threadIdx.x] = fetched_s;
+  };
+
+  if (first < last) fetch(first);
+  for (int t0 = first; t0 < last; t0 += kTile) {
+    const int count = min(kTile, last - t0);
+    __syncthreads();          // the tile before has been used by everybody
+    lay_down();
     __syncthreads();
+    if (t0 + kTile < last) fetch(t0 + kTile);
     for (int tt = 0; tt < count; ++tt) {
-      const float* qs = lds + static_cast<long>(tt) * token_floats + part * SP;
-      const float* ks = qs + array;
-      const float* gs = ks + array;
+      const float* qs = lds + tt * 3 * kArray + part * SP;
+      const float* ks = qs + kArray;
+      const float* gs = ks + kArray;
+      const float value = values[tt * kColumns + threadIdx.x / R], beta = scalars[2 * tt], kq = scalars[2 * tt + 1];
       float k[RP];
       float sum_k[4] = {0.f, 0.f, 0.f, 0.f}, sum_q[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -143,24 +223,25 @@ __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restric
           sum_q[e] = fmaf(S[i + e], qv[e], sum_q[e]);
         }
       }
-      float from_k = (sum_k[0] + sum_k[1]) + (sum_k[2] + sum_k[3]);
-      float from_q = (sum_q[0] + sum_q[1]) + (sum_q[2] + sum_q[3]);
-      for (int offset = R >> 1; offset > 0; offset >>= 1) {
-        from_k += __shfl_xor(from_k, offset, kWave);
-        from_q += __shfl_xor(from_q, offset, kWave);
-      }
-      const float u = scalars[2 * tt] * (values[tt * columns + threadIdx.x / R] - from_k);
+      const float from_k = column_sum<R>((sum_k[0] + sum_k[1]) + (sum_k[2] + sum_k[3]));
+      const float from_q = column_sum<R>((sum_q[0] + sum_q[1]) + (sum_q[2] + sum_q[3]));
+      const float u = beta * (value - from_k);
 #pragma unroll
       for (int i = 0; i < RP; ++i) S[i] = fmaf(k[i], u, S[i]);
-      if (part == 0 && works)
-        raw_out[(static_cast<long>(t0 + tt) * heads + h) * vdim + col] = fmaf(u, scalars[2 * tt + 1], from_q);
+      if (part == 0 && works) raw_out[(static_cast<long>(t0 + tt) * heads + h) * vdim + col] = fmaf(u, kq, from_q);
     }
   }
   if (works) {
 #pragma unroll
-    for (int i = 0; i < RP; ++i) {
+    for (int i = 0; i < RP; i += 4) {
       const int d = part * RP + i;
-      if (d < dim) kept[d] = S[i];
+      if (whole_fours && d < dim) {
+        *reinterpret_cast<float4*>(kept + d) = make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (d + e < dim) kept[d + e] = S[i + e];
+      }
     }
   }
 }
@@ -198,26 +279,31 @@ int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* be
   if (heads <= 0 || groups <= 0 || heads % groups != 0 || dim <= 0 || vdim <= 0 || dim > 2048) return -2;
   float* prepared = workspace;
   float* raw = workspace + static_cast<long>(tokens) * prepared_width(heads, groups, dim);
-  const int rp = dim <= 64 ? 8 : dim <= 256 ? 16 : 32;
+  const int rp = dim <= 256 ? 4 : dim <= 512 ? 8 : dim <= 1024 ? 16 : 32;
   int R = 1;
   while (R * rp < dim) R *= 2;
   const int columns = 256 / R, column_blocks = (vdim + columns - 1) / columns;
-  const long per_token = 3L * R * (rp + 4) + columns + 2;
-  const int tile = static_cast<int>(max(1L, min(16L, (48L * 1024 / 4) / per_token)));
-  const size_t lds = static_cast<size_t>(tile) * per_token * 4;
   const long v_at = 2L * groups * dim;
   const unsigned grid = static_cast<unsigned>(static_cast<long>(seqs) * heads * column_blocks);
   const long items = static_cast<long>(tokens) * heads;
-#define AKV_RECUR(RP)                                                                                                      \
-  delta_recur_kernel<T, RP><<<grid, 256, lds, stream>>>(prepared, static_cast<const T*>(conv), conv_stride, v_at, state,   \
-                                                        state_stride, q_start, seq_slots, raw, heads, groups, dim, vdim, R, tile)
+  const dim3 prepare_grid(static_cast<unsigned>(tokens), static_cast<unsigned>((groups + (heads * dim + 255) / 256 + 3) / 4));
+#define AKV_RECUR(RP, R_)                                                                                                   \
+  delta_recur_kernel<T, RP, R_><<<grid, 256, 0, stream>>>(prepared, static_cast<const T*>(conv), conv_stride, v_at, state, \
+                                                          state_stride, q_start, seq_slots, raw, heads, groups, dim, vdim)
   AKV_DISPATCH(dtype, T, {
-    delta_prepare_kernel<T><<<tokens, 256, 0, stream>>>(static_cast<const T*>(conv), conv_stride,
-                                                        static_cast<const T*>(beta_logits), beta_stride, decay_logits,
-                                                        decay_bias, rate, unit_eps, q_scale, prepared, heads, groups, dim);
-    if (rp == 8) AKV_RECUR(8);
-    else if (rp == 16) AKV_RECUR(16);
-    else AKV_RECUR(32);
+    delta_prepare_kernel<T><<<prepare_grid, 256, 0, stream>>>(static_cast<const T*>(conv), conv_stride,
+                                                              static_cast<const T*>(beta_logits), beta_stride, decay_logits,
+                                                              decay_bias, rate, unit_eps, q_scale, prepared, heads, groups, dim);
+    if (rp == 32) AKV_RECUR(32, 64);
+    else if (rp == 16) AKV_RECUR(16, 64);
+    else if (rp == 8) AKV_RECUR(8, 64);
+    else if (R == 64) AKV_RECUR(4, 64);
+    else if (R == 32) AKV_RECUR(4, 32);
+    else if (R == 16) AKV_RECUR(4, 16);
+    else if (R == 8) AKV_RECUR(4, 8);
+    else if (R == 4) AKV_RECUR(4, 4);
+    else if (R == 2) AKV_RECUR(4, 2);
+    else AKV_RECUR(4, 1);
     delta_finish_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(raw, norm_weight, gates, norm_eps,
                                                                                       static_cast<T*>(out), items, vdim);
   });
