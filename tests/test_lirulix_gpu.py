@@ -141,7 +141,7 @@ def random_configuration(seed: int) -> tuple:
     rng = random.Random(seed)
     layers = []
     for _ in range(rng.choice((2, 3, 4, 5))):
-        mlp = rng.choice((None, L.DENSE(rng.choice((40, 64, 100, 136)))))
+        mlp = rng.choice((None, L.DENSE(rng.choice((40, 64, 100, 132)))))
         kind = rng.choice(("attention", "attention_2", "channel_delta"))
         kv, group = rng.choice((1, 2, 3)), rng.choice((1, 2, 4, 5))
         dim = rng.choice((8, 12, 32, 64, 80))
@@ -161,7 +161,7 @@ def random_configuration(seed: int) -> tuple:
             mixer = L.DIFF(kv * group, kv, dim, vdim, rng.uniform(0.1, 0.5), L.ROT(dims, rng.choice((100.0, 1e4, 1e6)), scaling),
                            window, rng.choice((0.1, 0.3, 0.8)))
         layers.append(dict(type=kind, mlp=mlp, mixer=mixer))
-    raw = dict(architecture="Lirulix", vocab=rng.choice((97, 260, 1000)), width=rng.choice((40, 72, 96, 136, 192)),
+    raw = dict(architecture="Lirulix", vocab=rng.choice((97, 260, 1000)), width=rng.choice((40, 72, 96, 120, 192)),
                norm=dict(eps=rng.choice((1e-5, 1e-6))), layers=layers)
     if rng.random() < 0.7:
         start = rng.randrange(len(layers))
@@ -257,7 +257,7 @@ def test_attention_with_a_sink_alone(hip, dtype, heads, kv_heads, dim, vdim, dim
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,dims,page,window", [
-    (4, 2, 16, 12, 16, 4, 11), (3, 3, 24, 40, 8, 16, 16), (4, 2, 32, 64, 32, 16, 50), (2, 1, 64, 128, 16, 16, 136),
+    (4, 2, 16, 12, 16, 4, 11), (3, 3, 24, 40, 8, 16, 16), (4, 2, 32, 64, 32, 16, 50), (2, 1, 64, 128, 16, 16, 130),
     (2, 2, 8, 8, 8, 8, 1), (1, 1, 128, 32, 64, 32, None)])
 def test_differential_attention_alone(hip, dtype, heads, kv_heads, dim, vdim, dims, page, window):
     """The two maps of every head through rotation, cache and attention, then the difference, its norm and the gates,
