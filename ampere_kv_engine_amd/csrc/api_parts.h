@@ -109,13 +109,14 @@ int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const fl
 // q_scale; beta = sigmoid(beta_logits[t * beta_stride + h]); g = exp(-rate[h] * softplus(decay_logits[t, h, d] +
 // decay_bias[h, d])).  Per request and head, S [dim, vdim] (in the slot as [heads, vdim, dim] float32):
 // S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  out [tokens, heads x vdim] = o / rms(o) * norm_weight[i] *
-// sigmoid(gates[t, h, i]).  `workspace`: akv_delta_rule_workspace(...) floats.
+// sigmoid(gates[t, h, i]).  `workspace`: akv_delta_rule_workspace(...) floats.  `longest`: the most
+// tokens a request brings (chooses the walk's tile; the sums are the same either way).
 long akv_delta_rule_workspace(int tokens, int heads, int groups, int dim, int vdim);
 int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* beta_logits, long beta_stride,
                    const float* decay_logits, const float* decay_bias, const float* rate, const float* gates,
                    const float* norm_weight, float unit_eps, float norm_eps, float q_scale, float* state, long state_stride,
                    const int* q_start, const int* seq_slots, float* workspace, void* out, int tokens, int seqs, int heads,
-                   int groups, int dim, int vdim, hipStream_t stream);
+                   int groups, int dim, int vdim, int longest, hipStream_t stream);
 
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
 // down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the

@@ -11,7 +11,9 @@
 // nothing shortens, so what counts is a wave's instructions per token: with four rows a lane, one request's heads of
 // 128 x 128 are 1,024 waves - one on every vector unit of the device.  Since (g S + k u^T)^T q = (g S)^T q + u (k . q),
 // both sums are taken over the decayed state in one pass.  A tile of tokens' q, k and g passes through LDS for all columns
-// of the block; the next tile's values are asked for before this tile's tokens are walked.  `delta_finish` is token-wise
+// of the block; the next tile's values are asked for before this tile's tokens are walked; a whole tile is walked without a
+// loop (constant LDS addresses, a token's reads issued one token ahead) and its outputs are stored after the next tile's
+// barriers, which would otherwise wait for them.  `delta_finish` is token-wise
 // again: o / rms(o) times a weight per value channel and the sigmoid of a gate.  A request's state lies in its slot
 // transposed, [heads, vdim, dim]: a lane's rows of a column are consecutive floats.
 
@@ -101,29 +103,49 @@ template <int R> __device__ __forceinline__ float column_sum(float v) {
   return v;
 }
 
-// Tokens of a tile: what 48 KB of LDS hold of their q, k and g, 16 at most.
-template <int RP, int R> struct DeltaTile {
+// Tokens of a tile: what 48 KB of LDS hold of their q, k and g, CAP at most.  Every tile costs two barriers, its loads'
+// addresses and its stores: 32 tokens instead of 16 took an eighth off a long walk's time.  Steps of single tokens take
+// tiles of 4: many blocks of little LDS fit a compute unit and hide each other's loads of the state.
+template <int RP, int R, int CAP> struct DeltaTile {
   static constexpr int kSegment = RP == 4 ? 4 : RP + 4;     // (padding keeps the longer segments of neighbouring lanes in different banks)
   static constexpr int kArray = R * kSegment;
   static constexpr int kColumns = 256 / R;
-  static constexpr int kTokens = (12288 / (3 * kArray)) >= 16 ? 16 : (12288 / (3 * kArray)) >= 1 ? (12288 / (3 * kArray)) : 1;
+  static constexpr int kRoom = 12288 / (3 * kArray);
+  static constexpr int kTokens = kRoom >= CAP ? CAP : kRoom >= 16 ? 16 : kRoom >= 1 ? kRoom : 1;
   static constexpr int kFloats = kTokens * (3 * kArray + kColumns + 2);
+};
+
+// What a lane needs of one token: its RP rows of q, k and g, its column's value, the head's beta and k . q.
+template <int RP> struct TokenOperands {
+  float q[RP], k[RP], g[RP], value, beta, kq;
+  __device__ __forceinline__ void read(const float* qs, int array, const float* value_at, const float* scalar_at) {
+#pragma unroll
+    for (int i = 0; i < RP; i += 4) {
+      const float4 q4 = *reinterpret_cast<const float4*>(qs + i);
+      const float4 k4 = *reinterpret_cast<const float4*>(qs + array + i);
+      const float4 g4 = *reinterpret_cast<const float4*>(qs + 2 * array + i);
+      q[i] = q4.x, q[i + 1] = q4.y, q[i + 2] = q4.z, q[i + 3] = q4.w;
+      k[i] = k4.x, k[i + 1] = k4.y, k[i + 2] = k4.z, k[i + 3] = k4.w;
+      g[i] = g4.x, g[i + 1] = g4.y, g[i + 2] = g4.z, g[i + 3] = g4.w;
+    }
+    value = *value_at, beta = scalar_at[0], kq = scalar_at[1];
+  }
 };
 
 // A block: one request, one head, 256 / R columns of S.  Thread (column, part): rows part * RP .. part * RP + RP - 1.
 // LDS: per token of a tile three arrays (q, k, g) of R segments, then the tile's values [tile][columns] and its betas and
 // k . q [tile][2].
-template <typename T, int RP, int R>
+template <typename T, int RP, int R, int CAP>
 __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restrict__ prepared, const T* __restrict__ conv,
                                                           long conv_stride, long v_at, float* __restrict__ state,
                                                           long state_stride, const int* __restrict__ q_start,
                                                           const int* __restrict__ seq_slots, float* __restrict__ raw_out,
                                                           int heads, int groups, int dim, int vdim) {
-  using Tile = DeltaTile<RP, R>;
+  using Tile = DeltaTile<RP, R, CAP>;
   constexpr int SP = Tile::kSegment, kArray = Tile::kArray, kColumns = Tile::kColumns, kTile = Tile::kTokens;
   constexpr int kPadded = R * RP;
   constexpr int kVectorLoads = (kTile * kPadded + 255) / 256, kValueLoads = (kTile * kColumns + 255) / 256;
-  __shared__ float lds[Tile::kFloats];
+  __shared__ __attribute__((aligned(16))) float lds[Tile::kFloats];
   float* values = lds + kTile * 3 * kArray;        // [tile][columns]
   float* scalars = values + kTile * kColumns;      // [tile][2]: beta, k . q
   const int column_blocks = (vdim + kColumns - 1) / kColumns;
@@ -155,9 +177,32 @@ __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restric
   }
 
   // a tile's operands on their way from memory: asked for one tile ahead, laid into LDS when the tile before is done
-  float fetched_q[kVectorLoads], fetched_k[kVectorLoads], fetched_g[kVectorLoads], fetched_v[kValueLoads], fetched_s = 0.f;
+  // (with four rows a lane the segments lie in LDS without padding: where rows of the workspace allow 16-byte loads, four
+  // neighbouring floats travel together)
+  constexpr int kFourLoads = (kTile * kPadded / 4 + 255) / 256;
+  constexpr int kFetched = RP == 4 && 4 * kFourLoads > kVectorLoads ? 4 * kFourLoads : kVectorLoads;
+  const bool fours = RP == 4 && dim % 4 == 0 && width % 4 == 0 && (reinterpret_cast<uintptr_t>(prepared) & 15) == 0;
+  float fetched_q[kFetched], fetched_k[kFetched], fetched_g[kFetched], fetched_v[kValueLoads], fetched_s = 0.f;
+  // (loads are never skipped: a token or row that the tile does not have reads a neighbour's address, and what it read
+  // is replaced by a value without effect when the tile is laid down - no branch stands between a load and the walk)
+  int fetched_count = 0;
   auto fetch = [&](int t0) {
     const int count = min(kTile, last - t0);
+    fetched_count = count;
+    if (fours) {
+#pragma unroll
+      for (int j = 0; j < kFourLoads; ++j) {
+        const int index = threadIdx.x + j * 256;
+        const int tt = min(index / (kPadded / 4), count - 1), d = index % (kPadded / 4) * 4;
+        const float* row = prepared + static_cast<long>(t0 + tt) * width + (d < dim ? d : 0);
+        const float4 q4 = *reinterpret_cast<const float4*>(row + q_off);
+        const float4 k4 = *reinterpret_cast<const float4*>(row + k_off);
+        const float4 g4 = *reinterpret_cast<const float4*>(row + g_off);
+        fetched_q[4 * j] = q4.x, fetched_q[4 * j + 1] = q4.y, fetched_q[4 * j + 2] = q4.z, fetched_q[4 * j + 3] = q4.w;
+        fetched_k[4 * j] = k4.x, fetched_k[4 * j + 1] = k4.y, fetched_k[4 * j + 2] = k4.z, fetched_k[4 * j + 3] = k4.w;
+        fetched_g[4 * j] = g4.x, fetched_g[4 * j + 1] = g4.y, fetched_g[4 * j + 2] = g4.z, fetched_g[4 * j + 3] = g4.w;
+      }
+    } else {
 #pragma unroll
     for (int j = 0; j < kVectorLoads; ++j) {
       const int index = threadIdx.x + j * 256;
@@ -168,31 +213,80 @@ __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restric
       fetched_k[j] = real ? row[k_off + d] : 0.f;
       fetched_g[j] = real ? row[g_off + d] : 1.f;
     }
+    }
 #pragma unroll
     for (int j = 0; j < kValueLoads; ++j) {
       const int index = threadIdx.x + j * 256;
       const int tt = index / kColumns, c = col0 + index % kColumns;
-      fetched_v[j] = tt < count && c < vdim
-                         ? to_float(conv[static_cast<long>(t0 + tt) * conv_stride + v_at + static_cast<long>(h) * vdim + c]) : 0.f;
+      fetched_v[j] = to_float(conv[static_cast<long>(t0 + min(tt, count - 1)) * conv_stride + v_at + static_cast<long>(h) * vdim +
+                                   (c < vdim ? c : 0)]);
     }
-    const int which = threadIdx.x;
-    fetched_s = which < 2 * count ? prepared[static_cast<long>(t0 + which / 2) * width + b_off + (which & 1) * heads] : 0.f;
+    const int which = min(static_cast<int>(threadIdx.x), 2 * count - 1);
+    fetched_s = prepared[static_cast<long>(t0 + which / 2) * width + b_off + (which & 1) * heads];
   };
   auto lay_down = [&]() {
+    if (fours) {
 #pragma unroll
-    for (int j = 0; j < kVectorLoads; ++j) {
-      const int index = threadIdx.x + j * 256;
-      if (index >= kTile * kPadded) continue;
-      const int tt = index / kPadded, d = index % kPadded;
-      float* at = lds + tt * 3 * kArray + (d / RP) * SP + d % RP;
-      at[0] = fetched_q[j], at[kArray] = fetched_k[j], at[2 * kArray] = fetched_g[j];
+      for (int j = 0; j < kFourLoads; ++j) {
+        const int index = threadIdx.x + j * 256;
+        if (index >= kTile * kPadded / 4) continue;
+        float* at = lds + index / (kPadded / 4) * 3 * kArray + index % (kPadded / 4) * 4;
+        const bool real = index / (kPadded / 4) < fetched_count && index % (kPadded / 4) * 4 < dim;
+        const float4 zeros = make_float4(0.f, 0.f, 0.f, 0.f), ones = make_float4(1.f, 1.f, 1.f, 1.f);
+        *reinterpret_cast<float4*>(at) = real ? make_float4(fetched_q[4 * j], fetched_q[4 * j + 1], fetched_q[4 * j + 2], fetched_q[4 * j + 3]) : zeros;
+        *reinterpret_cast<float4*>(at + kArray) = real ? make_float4(fetched_k[4 * j], fetched_k[4 * j + 1], fetched_k[4 * j + 2], fetched_k[4 * j + 3]) : zeros;
+        *reinterpret_cast<float4*>(at + 2 * kArray) = real ? make_float4(fetched_g[4 * j], fetched_g[4 * j + 1], fetched_g[4 * j + 2], fetched_g[4 * j + 3]) : ones;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kVectorLoads; ++j) {
+        const int index = threadIdx.x + j * 256;
+        if (index >= kTile * kPadded) continue;
+        const int tt = index / kPadded, d = index % kPadded;
+        float* at = lds + tt * 3 * kArray + (d / RP) * SP + d % RP;
+        at[0] = fetched_q[j], at[kArray] = fetched_k[j], at[2 * kArray] = fetched_g[j];
+      }
     }
 #pragma unroll
     for (int j = 0; j < kValueLoads; ++j) {
       const int index = threadIdx.x + j * 256;
-      if (index < kTile * kColumns) values[index] = fetched_v[j];
+      if (index < kTile * kColumns)
+        values[index] = index / kColumns < fetched_count && col0 + index % kColumns < vdim ? fetched_v[j] : 0.f;
     }
-    if (threadIdx.x < 2 * kTile) scalars[threadIdx.x] = fetched_s;
+    if (threadIdx.x < 2 * kTile) scalars[threadIdx.x] = static_cast<int>(threadIdx.x) < 2 * fetched_count ? fetched_s : 0.f;
+  };
+
+  // one token: the state decays, takes the token's write and is read out; returns the column's output
+  auto walk = [&](const TokenOperands<RP>& now) {
+    float sum_k[4] = {0.f, 0.f, 0.f, 0.f}, sum_q[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RP; i += 4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[i + e] *= now.g[i + e];
+        sum_k[e] = fmaf(S[i + e], now.k[i + e], sum_k[e]);
+        sum_q[e] = fmaf(S[i + e], now.q[i + e], sum_q[e]);
+      }
+    }
+    const float from_k = column_sum<R>((sum_k[0] + sum_k[1]) + (sum_k[2] + sum_k[3]));
+    const float from_q = column_sum<R>((sum_q[0] + sum_q[1]) + (sum_q[2] + sum_q[3]));
+    const float u = now.beta * (now.value - from_k);
+#pragma unroll
+    for (int i = 0; i < RP; ++i) S[i] = fmaf(now.k[i], u, S[i]);
+    return fmaf(u, now.kq, from_q);
+  };
+
+  // A whole tile's outputs wait in registers and are stored after the next tile's barriers: a barrier waits for every
+  // store before it, and stores issued right before one would have the wave wait out their whole way to memory.
+  float outs[kTile];
+  int stored_from = -1;
+  auto store_tile = [&]() {
+    if (stored_from >= 0 && part == 0 && works) {
+      float* out_at = raw_out + (static_cast<long>(stored_from) * heads + h) * vdim + col;
+#pragma unroll
+      for (int tt = 0; tt < kTile; ++tt) out_at[static_cast<long>(tt) * heads * vdim] = outs[tt];
+    }
+    stored_from = -1;
   };
 
   if (first < last) fetch(first);
@@ -202,35 +296,34 @@ __global__ __launch_bounds__(256) void delta_recur_kernel(const float* __restric
     lay_down();
     __syncthreads();
     if (t0 + kTile < last) fetch(t0 + kTile);
-    for (int tt = 0; tt < count; ++tt) {
-      const float* qs = lds + tt * 3 * kArray + part * SP;
-      const float* ks = qs + kArray;
-      const float* gs = ks + kArray;
-      const float value = values[tt * kColumns + threadIdx.x / R], beta = scalars[2 * tt], kq = scalars[2 * tt + 1];
-      float k[RP];
-      float sum_k[4] = {0.f, 0.f, 0.f, 0.f}, sum_q[4] = {0.f, 0.f, 0.f, 0.f};
+    store_tile();
+    if (count == kTile) {
+      // a whole tile: its tokens one after the other without a loop around them - every LDS address is a constant and
+      // the tile's outputs leave in one go
+      TokenOperands<RP> ahead[2];
+      ahead[0].read(lds + part * SP, kArray, values + threadIdx.x / R, scalars);
 #pragma unroll
-      for (int i = 0; i < RP; i += 4) {
-        const float4 g4 = *reinterpret_cast<const float4*>(gs + i);
-        const float4 k4 = *reinterpret_cast<const float4*>(ks + i);
-        const float4 q4 = *reinterpret_cast<const float4*>(qs + i);
-        const float gv[4] = {g4.x, g4.y, g4.z, g4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w}, qv[4] = {q4.x, q4.y, q4.z, q4.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          S[i + e] *= gv[e];
-          k[i + e] = kv[e];
-          sum_k[e] = fmaf(S[i + e], kv[e], sum_k[e]);
-          sum_q[e] = fmaf(S[i + e], qv[e], sum_q[e]);
-        }
+      for (int tt = 0; tt < kTile; ++tt) {
+        // the next token's reads are issued before this token's sums and stay there: a wave alone on its vector unit has
+        // nobody to hide their way behind
+        if (tt + 1 < kTile)
+          ahead[(tt + 1) & 1].read(lds + (tt + 1) * 3 * kArray + part * SP, kArray,
+                                   values + (tt + 1) * kColumns + threadIdx.x / R, scalars + 2 * (tt + 1));
+        __builtin_amdgcn_sched_barrier(0);
+        outs[tt] = walk(ahead[tt & 1]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      const float from_k = column_sum<R>((sum_k[0] + sum_k[1]) + (sum_k[2] + sum_k[3]));
-      const float from_q = column_sum<R>((sum_q[0] + sum_q[1]) + (sum_q[2] + sum_q[3]));
-      const float u = beta * (value - from_k);
-#pragma unroll
-      for (int i = 0; i < RP; ++i) S[i] = fmaf(k[i], u, S[i]);
-      if (part == 0 && works) raw_out[(static_cast<long>(t0 + tt) * heads + h) * vdim + col] = fmaf(u, kq, from_q);
+      stored_from = t0;
+    } else {
+      for (int tt = 0; tt < count; ++tt) {
+        TokenOperands<RP> now;
+        now.read(lds + tt * 3 * kArray + part * SP, kArray, values + tt * kColumns + threadIdx.x / R, scalars + 2 * tt);
+        const float out = walk(now);
+        if (part == 0 && works) raw_out[(static_cast<long>(t0 + tt) * heads + h) * vdim + col] = out;
+      }
     }
   }
+  store_tile();
   if (works) {
 #pragma unroll
     for (int i = 0; i < RP; i += 4) {
@@ -274,7 +367,7 @@ int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* be
                    const float* decay_logits, const float* decay_bias, const float* rate, const float* gates,
                    const float* norm_weight, float unit_eps, float norm_eps, float q_scale, float* state, long state_stride,
                    const int* q_start, const int* seq_slots, float* workspace, void* out, int tokens, int seqs, int heads,
-                   int groups, int dim, int vdim, hipStream_t stream) {
+                   int groups, int dim, int vdim, int longest, hipStream_t stream) {
   if (tokens <= 0 || seqs <= 0) return 0;
   if (heads <= 0 || groups <= 0 || heads % groups != 0 || dim <= 0 || vdim <= 0 || dim > 2048) return -2;
   float* prepared = workspace;
@@ -287,9 +380,14 @@ int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* be
   const unsigned grid = static_cast<unsigned>(static_cast<long>(seqs) * heads * column_blocks);
   const long items = static_cast<long>(tokens) * heads;
   const dim3 prepare_grid(static_cast<unsigned>(tokens), static_cast<unsigned>((groups + (heads * dim + 255) / 256 + 3) / 4));
-#define AKV_RECUR(RP, R_)                                                                                                   \
-  delta_recur_kernel<T, RP, R_><<<grid, 256, 0, stream>>>(prepared, static_cast<const T*>(conv), conv_stride, v_at, state, \
-                                                          state_stride, q_start, seq_slots, raw, heads, groups, dim, vdim)
+#define AKV_RECUR_ARGS                                                                                                  \
+  prepared, static_cast<const T*>(conv), conv_stride, v_at, state, state_stride, q_start, seq_slots, raw, heads, groups, dim, \
+      vdim
+#define AKV_RECUR(RP, R_)                                                                                   \
+  do {                                                                                                      \
+    if (longest < 16) delta_recur_kernel<T, RP, R_, 4><<<grid, 256, 0, stream>>>(AKV_RECUR_ARGS);           \
+    else delta_recur_kernel<T, RP, R_, 32><<<grid, 256, 0, stream>>>(AKV_RECUR_ARGS);                       \
+  } while (0)
   AKV_DISPATCH(dtype, T, {
     delta_prepare_kernel<T><<<prepare_grid, 256, 0, stream>>>(static_cast<const T*>(conv), conv_stride,
                                                               static_cast<const T*>(beta_logits), beta_stride, decay_logits,
@@ -308,6 +406,7 @@ int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* be
                                                                                       static_cast<T*>(out), items, vdim);
   });
 #undef AKV_RECUR
+#undef AKV_RECUR_ARGS
   return AKV_LAUNCH_STATUS();
 }
 }

@@ -44,6 +44,83 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ x,
   out[static_cast<long>(n) * channels + c] = from_float<T>(SILU ? silu(acc) : acc);
 }
 
+// The same sums for eight neighbouring channels and TOK neighbouring tokens a thread, where the number of taps is one the
+// kernel is compiled for, channels come in eights and rows are 16-byte aligned: a row's eight inputs are one load and
+// serve every token of the thread that reaches back to them; the eight channels' weights are TAPS loads.  A token's
+// taps that lie before its request's portion come from the slot, as above.
+template <typename T> struct Eight {
+  static constexpr int kChunks = sizeof(T) * 8 / 16;
+  uint4 bits[kChunks];
+  __device__ __forceinline__ void load(const T* at) {
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) bits[i] = reinterpret_cast<const uint4*>(at)[i];
+  }
+  __device__ __forceinline__ void store(T* at) const {
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) reinterpret_cast<uint4*>(at)[i] = bits[i];
+  }
+  __device__ __forceinline__ float get(int i) const { return to_float(reinterpret_cast<const T*>(bits)[i]); }
+  __device__ __forceinline__ void set(int i, float v) { reinterpret_cast<T*>(bits)[i] = from_float<T>(v); }
+};
+
+template <typename T, typename TW, bool SILU, int TAPS, int TOK>
+__global__ __launch_bounds__(256) void conv_eights_kernel(const T* __restrict__ x, long x_stride, const TW* __restrict__ weight,
+                                                          const TW* __restrict__ bias, const float* __restrict__ state,
+                                                          long state_stride, long conv_at,
+                                                          const int* __restrict__ seq_of_token,
+                                                          const int* __restrict__ q_start, const int* __restrict__ seq_slots,
+                                                          T* __restrict__ out, int tokens, int channels) {
+  const int n0 = blockIdx.x * TOK;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c >= channels) return;
+  float w[TAPS][8];              // w[k][i]: tap k of channel c + i
+  {
+    Eight<TW> chunk[TAPS];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) chunk[j].load(weight + static_cast<long>(c) * TAPS + j * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int k = 0; k < TAPS; ++k) w[k][i] = chunk[(i * TAPS + k) / 8].get((i * TAPS + k) % 8);
+  }
+  float b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b[i] = bias != nullptr ? to_float(bias[c + i]) : 0.f;
+  Eight<T> rows[TOK + TAPS - 1];       // rows[j]: token n0 - (TAPS - 1) + j
+#pragma unroll
+  for (int j = 0; j < TOK + TAPS - 1; ++j) {
+    const int row = n0 - (TAPS - 1) + j;
+    if (row >= 0 && row < tokens) rows[j].load(x + static_cast<long>(row) * x_stride + c);
+  }
+#pragma unroll
+  for (int t = 0; t < TOK; ++t) {
+    const int n = n0 + t;
+    if (n >= tokens) break;
+    const int r = seq_of_token[n];
+    const int first = q_start[r];
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = b[i];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) {
+      const int row = n - (TAPS - 1 - k);
+      if (row >= first) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(w[k][i], rows[t + k].get(i), acc[i]);
+      } else {
+        const float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + conv_at
+                            + static_cast<long>(TAPS - 1 - (first - row)) * channels + c;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(w[k][i], kept[i], acc[i]);
+      }
+    }
+    Eight<T> result;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) result.set(i, SILU ? silu(acc[i]) : acc[i]);
+    result.store(out + static_cast<long>(n) * channels + c);
+  }
+}
+
 // After the convolution has read the old inputs: the slot keeps the last taps - 1 of (old inputs, the portion's).
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(const T* __restrict__ x, long x_stride,
@@ -204,12 +281,37 @@ int akv_conv_taps(const void* x, long x_stride, int dtype, const void* weight, c
   if (tokens <= 0) return 0;
   if (taps < 1 || channels <= 0 || activation < 0 || activation > 1) return -2;
   const dim3 grid(tokens, (channels + 255) / 256);
+  // eight channels a thread where rows, weights and outputs allow 16-byte accesses and the taps are among the compiled
+  // ones (a few tokens fill the device better with a thread a channel; both kernels sum in the same order)
+  const bool eights = tokens >= 32 && channels % 8 == 0 && x_stride % 8 == 0 && taps >= 2 && taps <= 5 &&
+                      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(weight) % 16 == 0;
+  const int per_thread = tokens >= 256 ? 4 : 1;
+  const dim3 grid_eights((tokens + per_thread - 1) / per_thread, (channels / 8 + 255) / 256);
+#define AKV_CONV_EIGHTS(T, TW, ACT, TAPS)                                                                                  \
+  do {                                                                                                                     \
+    if (per_thread == 4) conv_eights_kernel<T, TW, ACT, TAPS, 4><<<grid_eights, 256, 0, stream>>>(                         \
+        static_cast<const T*>(x), x_stride, static_cast<const TW*>(weight), static_cast<const TW*>(bias), state,           \
+        state_stride, conv_at, seq_of_token, q_start, seq_slots, static_cast<T*>(out), tokens, channels);                  \
+    else conv_eights_kernel<T, TW, ACT, TAPS, 1><<<grid_eights, 256, 0, stream>>>(                                         \
+        static_cast<const T*>(x), x_stride, static_cast<const TW*>(weight), static_cast<const TW*>(bias), state,           \
+        state_stride, conv_at, seq_of_token, q_start, seq_slots, static_cast<T*>(out), tokens, channels);                  \
+  } while (0)
+#define AKV_CONV_EIGHTS_TAPS(T, TW, ACT)                 \
+  do {                                                   \
+    if (taps == 2) AKV_CONV_EIGHTS(T, TW, ACT, 2);       \
+    else if (taps == 3) AKV_CONV_EIGHTS(T, TW, ACT, 3);  \
+    else if (taps == 4) AKV_CONV_EIGHTS(T, TW, ACT, 4);  \
+    else AKV_CONV_EIGHTS(T, TW, ACT, 5);                 \
+  } while (0)
 #define AKV_CONV_ARGS(T, TW)                                                                                         \
   static_cast<const T*>(x), x_stride, static_cast<const TW*>(weight), static_cast<const TW*>(bias), state, state_stride, \
       conv_at, seq_of_token, q_start, seq_slots, static_cast<T*>(out), channels, taps
 #define AKV_CONV(T, TW)                                                                          \
   do {                                                                                           \
-    if (activation == 1) conv_silu_kernel<T, TW, true><<<grid, 256, 0, stream>>>(AKV_CONV_ARGS(T, TW)); \
+    if (eights && activation == 1) AKV_CONV_EIGHTS_TAPS(T, TW, true);                            \
+    else if (eights) AKV_CONV_EIGHTS_TAPS(T, TW, false);                                         \
+    else if (activation == 1) conv_silu_kernel<T, TW, true><<<grid, 256, 0, stream>>>(AKV_CONV_ARGS(T, TW)); \
     else conv_silu_kernel<T, TW, false><<<grid, 256, 0, stream>>>(AKV_CONV_ARGS(T, TW));           \
   } while (0)
   if (dtype == kF32 && w_dtype == kF32) AKV_CONV(float, float);
@@ -218,6 +320,8 @@ int akv_conv_taps(const void* x, long x_stride, int dtype, const void* weight, c
   else return -1;
 #undef AKV_CONV
 #undef AKV_CONV_ARGS
+#undef AKV_CONV_EIGHTS_TAPS
+#undef AKV_CONV_EIGHTS
   return AKV_LAUNCH_STATUS();
 }
 

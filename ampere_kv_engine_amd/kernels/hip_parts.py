@@ -433,7 +433,8 @@ class PartsKernels:
             _ptr(conv), _long(width), self._code_of(conv), _ptr_at(beta_logits, beta_at), _long(beta_logits.shape[1]),
             _ptr(decay_logits), _ptr(decay_bias), _ptr(rate), _ptr(gates), _ptr(norm_weight), ctypes.c_float(unit_eps),
             ctypes.c_float(norm_eps), ctypes.c_float(q_scale), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start),
-            _ptr(ctx.seq_slots), _ptr(workspace), _ptr(out), tokens, ctx.num_seqs, heads, groups, dim, vdim, self._stream()),
+            _ptr(ctx.seq_slots), _ptr(workspace), _ptr(out), tokens, ctx.num_seqs, heads, groups, dim, vdim,
+            int(ctx.max_new_tokens) or tokens, self._stream()),
             "delta_rule")
 
     def _delta_workspace(self, need: int) -> torch.Tensor:

@@ -351,6 +351,34 @@ def test_delta_rule_kernels_alone(hip, dtype, heads, groups, dim, vdim, taps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("channels,extra,taps", [(64, 0, 4), (264, 8, 2), (40, 16, 3), (512, 24, 5), (48, 4, 4), (36, 4, 3), (16, 0, 6)])
+def test_convolution_over_long_and_short_steps(hip, dtype, channels, extra, taps):
+    """The convolution's kernel of eight channels a thread (rows of whole eights, 2 to 5 taps, steps of 32 tokens and
+    more; four tokens a thread from 256 tokens on) and the plain one, through steps whose portions begin in the middle
+    of a thread's tokens: a request's first taps come from its slot, never from the neighbouring request's rows."""
+    torch.manual_seed(channels + taps)
+    lengths = (700, 340)
+    rows = [(torch.randn(n, channels + extra) * 2).to(dtype).float() for n in lengths]
+    conv = (torch.randn(channels, taps) * 0.5).to(dtype)
+    state = torch.zeros(3, 5 + (taps - 1) * channels, dtype=torch.float32, device=DEVICE)
+    got = [torch.zeros(n, channels) for n in lengths]
+    for befores, counts in (((0, 0), (301, 2)), ((301, 2), (1, 1)), ((302, 3), (3, 326)), ((305, 329), (60, 2)), ((365, 331), (335, 9))):
+        ctx = _ctx(befores, counts)
+        projected = torch.cat([rows[r][b:b + c] for r, (b, c) in enumerate(zip(befores, counts))]).to(dtype).to(DEVICE)
+        conved = torch.empty(projected.shape[0], channels, dtype=dtype, device=DEVICE)
+        hip.conv_silu(projected, channels, conv.to(DEVICE), None, state, 0, ctx, conved, conv_at=5)
+        at = 0
+        for r, (b, c) in enumerate(zip(befores, counts)):
+            got[r][b:b + c] = conved[at:at + c].float().cpu()
+            at += c
+    assert (state[2] == 0.0).all() and (state[:2, :5] == 0.0).all()
+    for r, n in enumerate(lengths):
+        want = plain.silu(plain.causal_conv(rows[r][:, :channels], conv.float()))
+        error = (got[r] - want).abs().max() / want.abs().max()
+        assert error < (2e-6 if dtype == torch.float32 else 0.01), f"request {r}: {error:.2e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_token_wise_kernels(hip, dtype):
     """The normed embedding, the norm that takes a branch and a vector along, the gated activation."""
     torch.manual_seed(5)
