@@ -116,7 +116,8 @@ class CacheManager:
             if g.need.window is None:
                 return full
             span = g.need.window + (chunk if chunk is not None else num_tokens)
-            return min(full, (span + self.page_size - 1) // self.page_size + 1)
+            kept = (g.need.keep_first + self.page_size - 1) // self.page_size      # pages of the first tokens stay
+            return min(full, (span + self.page_size - 1) // self.page_size + 1 + kept)
         if group is not None:
             return one(group)
         return max((one(g) for g in self.groups), default=0)
@@ -145,7 +146,8 @@ class CacheManager:
             else:
                 state[slot].zero_()
         seq = Sequence(request_id, slot,
-                       [BlockTable(g.allocator, self.page_size, g.need.window, g.need.chunk) for g in self.groups])
+                       [BlockTable(g.allocator, self.page_size, g.need.window, g.need.chunk, g.need.keep_first)
+                        for g in self.groups])
         self._live[request_id] = seq
         return seq
 

@@ -5,7 +5,8 @@ Semantics follow the reference's pool and table (ampere_kv/block_pool.py:4-92): 
 `append_tokens` checks that every missing page is available before it takes any, `locate` refuses positions
 at or beyond the registered length, `release` gives everything back and may be called twice.  Beyond the
 reference: a table can give back, while the request lives, the pages that a window has passed or that belong to
-chunks of positions which no later query reads.
+chunks of positions which no later query reads - but never those of a request's first `keep_first` tokens, which
+stay visible behind the window.
 """
 
 from __future__ import annotations
@@ -51,15 +52,17 @@ class PageAllocator:
 class BlockTable:
     """One request's pages in one pool, in logical order, and the number of tokens registered."""
 
-    def __init__(self, allocator: PageAllocator, page_size: int, window: int | None = None, chunk: int | None = None):
+    def __init__(self, allocator: PageAllocator, page_size: int, window: int | None = None, chunk: int | None = None,
+                 keep_first: int = 0):
         self._allocator = allocator
         self.page_size = page_size
         self.window = window
         self.chunk = chunk        # queries read keys of their own chunk of so many positions only (counted from 0)
+        self.kept_pages = (max(int(keep_first), 0) + page_size - 1) // page_size      # never given back while it lives
         self._pages: list[int] = []
         self._mirror = np.empty(16, dtype=np.int32)   # the same ids as an array, for the step's metadata
         self._length = 0
-        self._first_live = 0      # logical index of the first page not yet given back
+        self._first_live = self.kept_pages      # logical index of the first page, after the kept ones, not yet given back
         self._changed: list[int] = []   # entries that changed since `take_changes` (what a device copy must be told)
 
     def take_changes(self) -> list[tuple[int, int]]:
@@ -88,7 +91,7 @@ class BlockTable:
 
     @property
     def num_held(self) -> int:
-        return len(self._pages) - self._first_live
+        return min(len(self._pages), self.kept_pages) + max(len(self._pages) - self._first_live, 0)
 
     def _passed_pages(self, next_position: int) -> int:
         """Live pages that lie wholly before the oldest key a query at `next_position` may read."""
@@ -144,9 +147,9 @@ class BlockTable:
         return page, offset
 
     def release(self) -> None:
-        for page in self._pages[self._first_live:]:
+        for page in self._pages[:self.kept_pages] + self._pages[max(self._first_live, self.kept_pages):]:
             self._allocator.free(page)
         self._pages.clear()
         self._changed.clear()
         self._length = 0
-        self._first_live = 0
+        self._first_live = self.kept_pages

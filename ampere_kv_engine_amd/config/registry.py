@@ -14,6 +14,7 @@ from typing import Protocol
 
 from .keranex import KeranexConfig
 from .lirulix import LirulixConfig
+from .mekuvik import MekuvikConfig
 from .qwen3 import ConfigError, Qwen3Config
 from .tukevik import TukevikConfig
 from .specs import ModelSpec
@@ -67,3 +68,4 @@ register_architecture(Qwen3Config.architecture, Qwen3Config)
 register_architecture(KeranexConfig.architecture, KeranexConfig)
 register_architecture(TukevikConfig.architecture, TukevikConfig)
 register_architecture(LirulixConfig.architecture, LirulixConfig)
+register_architecture(MekuvikConfig.architecture, MekuvikConfig)

@@ -52,12 +52,14 @@ class RunEntry:
     for an entry that only reads what another entry wrote.  A layer that runs several times with the same weights
     and a cache or state of its own each time names the time in `cache_copy` (0, 1, ...): every (cache_layer,
     cache_copy) is a cache of its own.  `adds_row`: before this entry runs, row `adds_row` of the model's table of
-    vectors (`ModelSpec.pass_vectors`) is added to every token's residual sum."""
+    vectors (`ModelSpec.pass_vectors`) is added to every token's residual sum.  `adds_embedding`: before this entry runs,
+    the embedding's output - the residual sum as it was before the first layer - is added to it."""
     layer: int
     cache_layer: int
     writes_cache: bool = True
     cache_copy: int = 0
     adds_row: int | None = None
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

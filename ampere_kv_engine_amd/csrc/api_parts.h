@@ -19,10 +19,21 @@ int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots
                         hipStream_t stream);
 // stream [tokens, hidden] float32.  With `delta` (dtype): stream += delta / rms(delta) * post_weight (or += delta where
 // post_weight is null: stream += delta_scale * delta).  With `offset` [hidden]: stream += offset, every row, after the
-// branch.  With `out` (dtype): out = stream / rms(stream) * pre_weight, rounded once.
+// branch.  With `out` (dtype): out = stream / rms(stream) * pre_weight, rounded once.  With `delta2` (dtype; only beside a
+// `delta` that is not normed): stream += delta_scale * (delta + delta2) - two branches that read the same input.
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      float delta_scale, const float* offset, hipStream_t stream);
+                      float delta_scale, const float* offset, const void* delta2, hipStream_t stream);
+// out[n] = table[id] (with `accumulate`: out[n] += table[id]), float32; an id of -1: the token chosen last for the row's
+// request, where the slot words are given
+int akv_embed_rows(const int* ids, const void* table, int dtype, float* out, int tokens, int hidden, int vocab, int accumulate,
+                   const int* seq_of_token, const int* seq_slots, const int* slot_words, hipStream_t stream);
+// x [tokens, width] (x_dtype: float32 or `dtype`) at x_stride per token -> out (dtype) at out_stride per token =
+// x / rms(x over the whole row) * weight (where `normed`; `weight` may be null) * act(gates[t * gate_stride + i]) * out_scale;
+// gate_act 0: no gate, 1: sigmoid, 2: silu
+int akv_norm_gate_rows(const void* x, int x_dtype, long x_stride, int width, int normed, const float* weight, float eps,
+                       const void* gates, long gate_stride, int gate_act, void* out, int dtype, long out_stride,
+                       float out_scale, long tokens, hipStream_t stream);
 // out[n] = table[id] / rms(table[id]) * weight: the start of a residual sum that is normed before the first layer (an id
 // of -1: the token chosen last for the row's request, where the slot words are given)
 int akv_embed_normed(const int* ids, const void* table, int dtype, const float* weight, float eps, float* out, int tokens,
@@ -49,13 +60,17 @@ int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, v
 // `maps` > 1: a head's queries and keys are `maps` vectors of `dim` side by side (rows [q (q_heads x maps x dim) | k (kv_heads
 // x maps x dim) | v]), each normed and rotated for itself; key pages [pages, kv_heads, page, maps x dim].  `table`
 // [table_positions, rot_dims / 2, 2] (cos, sin; null: no rotation): a vector's first rot_dims dimensions are rotated by the
-// token's position, dimension i with i + rot_dims / 2.
+// token's position, dimension i with i + rot_dims / 2 (`interleaved`: dimension 2 i with 2 i + 1).  `whole`: the root mean
+// square is taken over all query vectors of the token at once, and over all its key vectors.  `q_weight` [q_heads x maps x
+// dim], `k_weight` [kv_heads x maps x dim] (float32, may be null): multiplied in after the norm, before the rotation.
 int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
                         int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
                         long num_pages, void* q_out, int maps, const float* table, int table_positions, int rot_dims,
-                        const int* positions, hipStream_t stream);
+                        const int* positions, const float* q_weight, const float* k_weight, int whole, int interleaved,
+                        hipStream_t stream);
 // out [tokens, q_heads, vdim].  score = (q . k) * scale, then softcap * tanh(score / softcap) where softcap > 0; a query at
-// position p sees the keys j <= p with j > p - window (window > 0) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
+// position p sees the keys j <= p with j > p - window (window > 0; the request's first `keep_first` keys stay visible
+// behind the window) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
 // with `sink` the softmax's denominator has one more term exp(0); with `gates` head h's output is multiplied by
 // sigmoid(gates[t * gate_stride + gate_at + h]).  A token's outputs lie at out + t * out_stride, times out_scale.
 // `row_waves` (1 .. 16) waves share a token's head: each takes every row_waves-th tile of 64 keys.  `sink_logits` [q_heads]
@@ -66,7 +81,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
                              int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
-                             const float* sink_logits, int maps, hipStream_t stream);
+                             const float* sink_logits, int maps, int keep_first, hipStream_t stream);
 
 // The same for rows first_row .. tokens - 1 of a bfloat16 step, on the matrix cores: keys and values 32, 64, 128 or 256
 // wide, pages of a multiple of 16 tokens (-2 otherwise); a request's rows follow each other in the order of their positions.
@@ -75,25 +90,27 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
                               float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
-                              const float* sink_logits, int maps, hipStream_t stream);
+                              const float* sink_logits, int maps, int keep_first, hipStream_t stream);
 
 // ---- mixers with a state of fixed size (recurrent_mixers.hip) ----------------------------------------------------------
 // projected [tokens, stride]: rows [q | k (heads x dim each) | v | g (heads x vdim each)].  q and k are rotated over their
 // first rot_dims dimensions (pairs i, i + rot_dims / 2; `table` [positions, rot_dims / 2, 2] holds cos and sin), k times
 // key_scale; per request and head S [dim, vdim] (at state[slot * state_stride + head * dim * vdim]) <- decay S + k v^T,
 // o = S^T q; out [tokens, heads, vdim] (a token's at out + t * out_stride) = o / rms(o) * silu(g) * out_scale.
+// `input_act` 1: q, k and v pass silu as they are read.  `raw` [tokens, heads, vdim] float32 (may be null): the outputs o
+// are left there as they are and `out` is not written - for a caller that norms and gates all heads together.
 int akv_retention(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                   const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
                   long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
-                  long out_stride, float out_scale, hipStream_t stream);
+                  long out_stride, float out_scale, int input_act, float* raw, hipStream_t stream);
 // The same with every request's tokens cut into chunks of `length` that are worked on side by side - sums of k v^T per
 // chunk, the states before the chunks one after the other, then every chunk's outputs: `sums` holds 2 * seqs * heads *
 // chunks * dim * vdim floats, chunks = the most chunks a request of the step has.
 int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                           const float* table, int table_positions, float key_scale, const float* decay, float eps,
                           float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
-                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks,
-                          hipStream_t stream);
+                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks, int input_act,
+                          float* raw, hipStream_t stream);
 // u [tokens, channels]; gates [tokens, blocks, 2 * channels / blocks] float32 (a block's recurrence-gate logits, then its
 // input-gate logits) before their biases `gate_bias` [blocks, 2 * channels / blocks]; a = exp(rate[c] * sigmoid(.));
 // S [channels] at the start of a slot's state <- a S + sqrt(1 - a^2) sigmoid(.) u; out = S * gelu_tanh(y), y at
@@ -121,15 +138,17 @@ int akv_delta_rule(const void* conv, long conv_stride, int dtype, const void* be
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
 // down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the
 // shared key part rotated (first `rot_dims` of its `rot` dimensions) into the token's record [kv_rank + rot].  With
-// `latents_t` [pages, kv_rank, page_size] the normed latent is written there too, keys contiguous.
+// `latents_t` [pages, kv_rank, page_size] the normed latent is written there too, keys contiguous.  Rotation pairs are
+// dimensions (i, i + rot_dims / 2), or (2 i, 2 i + 1) with `interleaved`.  `down_stride`: elements from one token's row of
+// `down` to the next (0: the rows hold nothing else).
 int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
                       const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
                       const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
-                      void* latents_t, int page_size, hipStream_t stream);
+                      void* latents_t, int page_size, int interleaved, long down_stride, hipStream_t stream);
 // q [tokens, heads, dim + rot] -> q_abs[..., at : at + rot] (float32 or bfloat16, row width `width`), rotated by position
 int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
                        const float* table, int table_positions, const int* positions, void* q_abs, int out_dtype,
-                       int width, int at, hipStream_t stream);
+                       int width, int at, int interleaved, hipStream_t stream);
 // y[t, h, j] = sum_i x[t, h, i] * w[h, i, j]   (w [heads, ins, outs]; x and y addressed by token and head strides)
 int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_head_stride, const void* w, int w_dtype,
                      void* y, int y_dtype, long y_token_stride, long y_head_stride, int tokens, int heads, int ins,
@@ -178,8 +197,14 @@ int akv_selective_scan(const void* x, int dtype, float* dt, const float* bc, con
 int akv_route(const float* logits, float* gates, int tokens, int experts, int top, int groups, int keep,
               hipStream_t stream);
 // logits [tokens, scored] -> gates: the `top` largest of the first `experts` logits get the softmax over themselves, the
-// other experts 0, every further column its sigmoid
-int akv_route_chosen(const float* logits, float* gates, int tokens, int experts, int scored, int top, hipStream_t stream);
+// other experts 0, every further column its sigmoid.  `law` 1: logits [tokens, experts]; a chosen expert's gate is the
+// sigmoid of its own logit, and every further column of gates [tokens, scored] becomes 1
+int akv_route_chosen(const float* logits, float* gates, int tokens, int experts, int scored, int top, int law,
+                     hipStream_t stream);
+// act[t, c] = f(gates[t, e(c)] * up[t, c]) (`inside`) or gates[t, e(c)] * f(up[t, c]); f 0: gelu (erf), 1: gelu (tanh), 2: silu,
+// 3: relu squared; e(c) = c / ff below experts * ff, else `experts`
+int akv_gate_activation(const void* up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
+                        int columns, int scored, int kind, int inside, hipStream_t stream);
 // act[t, c] = gates[t, e(c)] * silu(gate_up[t, c]) * gate_up[t, columns + c]; e(c) = c / ff below experts * ff, else `experts`
 int akv_gate_silu_mul(const void* gate_up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
                       int columns, int scored, hipStream_t stream);

@@ -25,7 +25,10 @@ __device__ __forceinline__ void wave_sync_lds() {
 // With `maps` > 1 a head's queries and keys are `maps` vectors of `dim` side by side: the token has q_heads * maps query
 // vectors and kv_heads * maps key vectors, each normed and rotated for itself, and a key head's record in the pages is
 // its `maps` vectors one after the other.  With `table` [positions, rot_dims / 2, 2] (cos, sin) a vector's first rot_dims
-// dimensions are rotated by the token's position, dimension i with i + rot_dims / 2.
+// dimensions are rotated by the token's position, dimension i with i + rot_dims / 2 - or, with `interleaved`, dimension 2 i
+// with 2 i + 1.  With `whole` the root mean square is taken over all of the token's query vectors at once (and over all of
+// its key vectors): every wave sums its side's whole projection for itself.  `q_weight` [q vectors x dim] and `k_weight`
+// [k vectors x dim] (float32, either may be null) multiply the normed values, before the rotation.
 template <typename T>
 __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restrict__ projected, long stride, long tokens,
                                                               int q_heads, int kv_heads, int dim, int vdim, float eps,
@@ -33,7 +36,10 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
                                                               T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
                                                               long num_pages, T* __restrict__ q_out, int maps,
                                                               const float* __restrict__ table, int table_positions,
-                                                              int rot_dims, const int* __restrict__ positions) {
+                                                              int rot_dims, const int* __restrict__ positions,
+                                                              const float* __restrict__ q_weight,
+                                                              const float* __restrict__ k_weight, int whole,
+                                                              int interleaved) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const int q_vectors = q_heads * maps, k_vectors = kv_heads * maps;
   const int items = q_vectors + k_vectors + kv_heads;
@@ -58,27 +64,32 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
     }
     float scale = 1.f;
     if (normed) {
+      const T* side = whole ? row + (is_q ? 0L : static_cast<long>(q_vectors) * dim) : x;
+      const int count = whole ? (is_q ? q_vectors : k_vectors) * dim : dim;
       float squares = 0.f;
-      for (int i = lane; i < dim; i += kWave) {
-        const float v = to_float(x[i]);
+      for (int i = lane; i < count; i += kWave) {
+        const float v = to_float(side[i]);
         squares += v * v;
       }
-      scale = rsqrtf(wave_sum(squares) / static_cast<float>(dim) + eps);
+      scale = rsqrtf(wave_sum(squares) / static_cast<float>(count) + eps);
     }
+    const float* gain = is_q ? q_weight : k_weight;
+    if (gain != nullptr) gain += static_cast<long>(is_q ? which : which - q_vectors) * dim;
     if (table == nullptr || rot_dims <= 0) {
-      for (int i = lane; i < dim; i += kWave) y[i] = from_float<T>(to_float(x[i]) * scale);
+      for (int i = lane; i < dim; i += kWave) y[i] = from_float<T>(to_float(x[i]) * scale * (gain != nullptr ? gain[i] : 1.f));
     } else {
       const int half = rot_dims / 2;
       const int pos = positions[n];
       const bool known = pos >= 0 && pos < table_positions;      // (a position beyond the table poisons the vector)
       const float* angles = table + static_cast<long>(known ? pos : 0) * half * 2;
       for (int i = lane; i < dim; i += kWave) {
-        float v = to_float(x[i]) * scale;
+        float v = to_float(x[i]) * scale * (gain != nullptr ? gain[i] : 1.f);
         if (i < rot_dims) {
-          const bool low = i < half;
-          const int pair = low ? i : i - half;
+          const bool low = interleaved ? (i & 1) == 0 : i < half;
+          const int pair = interleaved ? i >> 1 : (low ? i : i - half);
+          const int mate = interleaved ? i ^ 1 : (low ? i + half : i - half);
           const float c = angles[2 * pair], s = angles[2 * pair + 1];
-          const float other = to_float(x[low ? i + half : i - half]) * scale;
+          const float other = to_float(x[mate]) * scale * (gain != nullptr ? gain[mate] : 1.f);
           v = low ? v * c - other * s : v * c + other * s;
           if (!known) v = __uint_as_float(0x7fc00000u);
         }
@@ -127,7 +138,8 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
     long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
     const int* __restrict__ block_table, const int* __restrict__ table_rows, int table_width, T* __restrict__ out,
     long tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-    int chunk, int window, int sink, long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps) {
+    int chunk, int window, int sink, long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps,
+    int keep_first) {
   // (`q_heads` counts query vectors: with `maps` > 1 a head has `maps` of them, which read the `maps` vectors of their key
   // head's record in turn and the same values; vector v's key head is still v / (q_heads / kv_heads))
   extern __shared__ unsigned char lds_raw[];
@@ -164,9 +176,13 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
 #pragma unroll
     for (int c = 0; c < kMaxValueRegs; ++c) acc[g][c] = 0.f;
   }
-  for (int tile = lowest / kWave + wave; tile * kWave <= pos; tile += kRowWaves) {
+  // the request's first `keep_first` keys stay visible behind the window: their tiles come first, then the window's
+  const int first_tile = lowest / kWave, kept_tiles = min((keep_first + kWave - 1) / kWave, first_tile);
+  const int all_tiles = kept_tiles + pos / kWave - first_tile + 1;
+  for (int turn = wave; turn < all_tiles; turn += kRowWaves) {
+    const int tile = turn < kept_tiles ? turn : first_tile + turn - kept_tiles;
     const int j = tile * kWave + lane;
-    const bool valid = j >= lowest && j <= pos;
+    const bool valid = (j >= lowest || j < keep_first) && j <= pos;
     float s[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) s[g] = -INFINITY;
@@ -343,7 +359,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
     const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ block_table,
     const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, int first_row, int tokens, int q_heads,
     int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink,
-    long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps) {
+    long out_stride, float out_scale, const float* __restrict__ sink_logits, int maps, int keep_first) {
   constexpr int DIM = 32 * DT, VDIM = 16 * VT;
   extern __shared__ float tile_shares[];      // [waves][2 + 4 VT][64]: what the block's waves found over their keys
   // a block is 16 rows and a head; its waves take the steps of 16 keys in turn
@@ -404,10 +420,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
       for (int vt = 0; vt < VT; ++vt) vs[vt] = load_bf16x4(vp + static_cast<long>(vt) * 16 * page_size);
       return true;
     };
-    const int j_first = (lo_run & ~15) + wave * 16, j_step = waves * 16;
-    if (j_first <= p_last) there = fetch(j_first, keys, values);
-    for (int j0 = j_first; j0 <= p_last; j0 += j_step) {
-      there_next = j0 + j_step <= p_last ? fetch(j0 + j_step, keys_next, values_next) : false;
+    // steps of 16 keys: those of the request's first `keep_first` keys that lie before the window, then the window's
+    const int first_step = lo_run >> 4, kept_steps = min((keep_first + 15) >> 4, first_step);
+    const int all_steps = kept_steps + (p_last >> 4) - first_step + 1;
+    auto keys_of = [&](int turn) { return (turn < kept_steps ? turn : first_step + turn - kept_steps) << 4; };
+    if (wave < all_steps) there = fetch(keys_of(wave), keys, values);
+    for (int turn = wave; turn < all_steps; turn += waves) {
+      const int j0 = keys_of(turn);
+      there_next = turn + waves < all_steps ? fetch(keys_of(turn + waves), keys_next, values_next) : false;
       if (there) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -424,7 +444,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <=
             const float e = __expf(2.f * fabsf(v) * inverse_cap);
             v = copysignf(softcap * (1.f - 2.f * __frcp_rn(e + 1.f)), v);
           }
-          s[i] = (in_run && j >= my_lowest && j <= my_pos) ? v : -INFINITY;
+          s[i] = (in_run && (j >= my_lowest || j < keep_first) && j <= my_pos) ? v : -INFINITY;
           highest = fmaxf(highest, s[i]);
         }
         highest = fmaxf(highest, __shfl_xor(highest, 16, kWave));
@@ -525,7 +545,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
                               float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
-                              const float* sink_logits, int maps, hipStream_t stream) {
+                              const float* sink_logits, int maps, int keep_first, hipStream_t stream) {
   if (tokens <= first_row) return 0;
   if (page_size % 16 != 0 || q_heads % kv_heads != 0 || maps < 1) return -2;
   const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
@@ -537,7 +557,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages),         \
       static_cast<const bf16_t*>(gates), gate_stride, gate_at, seq_of_token, q_start, positions, block_table, table_rows, \
       table_width, static_cast<bf16_t*>(out), first_row, tokens, q_heads, kv_heads, page_size, num_pages, scale, softcap, \
-      chunk, window, sink, out_stride, out_scale, sink_logits, maps)
+      chunk, window, sink, out_stride, out_scale, sink_logits, maps, keep_first)
 #define AKV_TILES_V(DT)                    \
   switch (vdim) {                          \
     case 32: AKV_TILES(DT, 2); break;      \
@@ -561,7 +581,8 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
 int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
                         int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
                         long num_pages, void* q_out, int maps, const float* table, int table_positions, int rot_dims,
-                        const int* positions, hipStream_t stream) {
+                        const int* positions, const float* q_weight, const float* k_weight, int whole, int interleaved,
+                        hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || maps < 1) return -2;
   if (table != nullptr && (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > dim || positions == nullptr)) return -2;
@@ -569,7 +590,8 @@ int akv_unit_norm_write(const void* projected, long stride, int dtype, long toke
   AKV_DISPATCH(dtype, T, unit_norm_write_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(
                              static_cast<const T*>(projected), stride, tokens, q_heads, kv_heads, dim, vdim, eps, normed,
                              slot_map, static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages,
-                             static_cast<T*>(q_out), maps, table, table_positions, rot_dims, positions));
+                             static_cast<T*>(q_out), maps, table, table_positions, rot_dims, positions, q_weight,
+                             k_weight, whole, interleaved));
   return AKV_LAUNCH_STATUS();
 }
 
@@ -578,7 +600,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
                              int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
-                             const float* sink_logits, int maps, hipStream_t stream) {
+                             const float* sink_logits, int maps, int keep_first, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (maps < 1) return -2;
   const int kRowWaves = row_waves;
@@ -610,7 +632,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                    static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),            \
                    static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows, \
                    table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale, \
-                   softcap, chunk, window, sink, out_stride, out_scale, sink_logits, maps))
+                   softcap, chunk, window, sink, out_stride, out_scale, sink_logits, maps, keep_first))
 #define AKV_ROWS_G(VEC)          \
   switch (bundle) {              \
     case 4: AKV_ROWS(VEC, 4); break; \

@@ -25,12 +25,11 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
     const T* __restrict__ down, int q_rank, int kv_rank, int rot, int rot_dims, const float* __restrict__ q_weight,
     const float* __restrict__ kv_weight, float eps, const float* __restrict__ table, int table_positions,
     const int* __restrict__ positions, const int* __restrict__ slot_map, T* __restrict__ cq, T* __restrict__ records,
-    long record_slots, T* __restrict__ latents_t, int page_size) {
+    long record_slots, T* __restrict__ latents_t, int page_size, int interleaved, long down_stride) {
   __shared__ float scratch[16];
   const int n = blockIdx.x;
   const bool writes = records != nullptr;
-  const int width = q_rank + (writes ? kv_rank + rot : 0);
-  const T* src = down + static_cast<size_t>(n) * width;
+  const T* src = down + static_cast<size_t>(n) * down_stride;
   float acc = 0.f;
   for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
     const float v = to_float(src[i]);
@@ -68,10 +67,12 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
     } else if (!known) {
       value = __uint_as_float(kPoison);
     } else {
-      const int j = i < half ? i : i - half;
+      // pair j is dimensions (j, j + half), or (2 j, 2 j + 1) where the pairs are interleaved
+      const int j = interleaved ? i >> 1 : (i < half ? i : i - half);
+      const bool low = interleaved ? (i & 1) == 0 : i < half;
       const float c = table[(static_cast<size_t>(pos) * half + j) * 2], s = table[(static_cast<size_t>(pos) * half + j) * 2 + 1];
-      const float u = to_float(key[j]), v = to_float(key[j + half]);
-      value = i < half ? u * c - v * s : v * c + u * s;
+      const float u = to_float(key[interleaved ? 2 * j : j]), v = to_float(key[interleaved ? 2 * j + 1 : j + half]);
+      value = low ? u * c - v * s : v * c + u * s;
     }
     record[kv_rank + i] = from_float<T>(value);
   }
@@ -81,7 +82,8 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
 template <typename T, typename TY>
 __global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int heads, int dim, int rot, int rot_dims,
                                       const float* __restrict__ table, int table_positions,
-                                      const int* __restrict__ positions, TY* __restrict__ q_abs, int width, int at) {
+                                      const int* __restrict__ positions, TY* __restrict__ q_abs, int width, int at,
+                                      int interleaved) {
   const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (index >= tokens * heads * rot) return;
   const int i = static_cast<int>(index % rot);
@@ -97,10 +99,11 @@ __global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int 
     if (pos < 0 || pos >= table_positions) {
       value = __uint_as_float(kPoison);
     } else {
-      const int j = i < half ? i : i - half;
+      const int j = interleaved ? i >> 1 : (i < half ? i : i - half);
+      const bool low = interleaved ? (i & 1) == 0 : i < half;
       const float c = table[(static_cast<size_t>(pos) * half + j) * 2], s = table[(static_cast<size_t>(pos) * half + j) * 2 + 1];
-      const float u = to_float(src[j]), v = to_float(src[j + half]);
-      value = i < half ? u * c - v * s : v * c + u * s;
+      const float u = to_float(src[interleaved ? 2 * j : j]), v = to_float(src[interleaved ? 2 * j + 1 : j + half]);
+      value = low ? u * c - v * s : v * c + u * s;
     }
   }
   q_abs[row * width + at + i] = from_float<TY>(value);
@@ -726,19 +729,22 @@ extern "C" {
 int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
                       const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
                       const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
-                      void* latents_t, int page_size, hipStream_t stream) {
+                      void* latents_t, int page_size, int interleaved, long down_stride, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  const long needed = q_rank + (records != nullptr ? kv_rank + rot : 0);
+  if (down_stride == 0) down_stride = needed;
+  if (down_stride < needed) return -2;
   if (rot_dims % 2 || rot_dims > rot || q_rank <= 0 || (latents_t != nullptr && page_size <= 0)) return -2;
   AKV_DISPATCH(dtype, T, latent_encode_kernel<T><<<tokens, 256, 0, stream>>>(
                              static_cast<const T*>(down), q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table,
                              table_positions, positions, slot_map, static_cast<T*>(cq), static_cast<T*>(records),
-                             record_slots, static_cast<T*>(latents_t), page_size));
+                             record_slots, static_cast<T*>(latents_t), page_size, interleaved, down_stride));
   return AKV_LAUNCH_STATUS();
 }
 
 int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
                        const float* table, int table_positions, const int* positions, void* q_abs, int out_dtype,
-                       int width, int at, hipStream_t stream) {
+                       int width, int at, int interleaved, hipStream_t stream) {
   const long count = tokens * heads * rot;
   if (count <= 0) return 0;
   if (rot_dims % 2 || rot_dims > rot || at + rot > width) return -2;
@@ -746,11 +752,11 @@ int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim
   if (out_dtype == kF32) {
     AKV_DISPATCH(dtype, T, rotate_queries_kernel<T, float><<<blocks, 256, 0, stream>>>(
                                static_cast<const T*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
-                               static_cast<float*>(q_abs), width, at));
+                               static_cast<float*>(q_abs), width, at, interleaved));
   } else if (out_dtype == kBF16 && dtype == kBF16) {
     rotate_queries_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>(
         static_cast<const bf16_t*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
-        static_cast<bf16_t*>(q_abs), width, at);
+        static_cast<bf16_t*>(q_abs), width, at, interleaved);
   } else {
     return -1;
   }

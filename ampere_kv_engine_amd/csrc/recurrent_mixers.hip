@@ -1,6 +1,7 @@
 // Mixers whose requests carry a float32 state of fixed size from token to token:
 //   retention - S [dim, vdim] per head, S <- decay S + k v^T, o = S^T q, with rotary positions on q and k, the unit norm of o
-//   per head and the gate silu(g) in the same kernel;
+//   per head and the gate silu(g) in the same kernel - or, for a mixer that norms and gates all heads together, the raw
+//   outputs in float32 for a kernel of its own; q, k and v may pass silu as they are read (`input_act`);
 //   a gated linear recurrence - S [channels], S <- a S + sqrt(1 - a^2) i u with a = exp(rate r), r and i sigmoids of
 //   block-diagonal products, the output S * gelu_tanh(y).
 // Everything but the loads of the projections is float32.  A request's tokens are taken in the order of their positions
@@ -28,7 +29,8 @@ __global__ __launch_bounds__(1024) void retention_kernel(
     const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
     const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay, float eps,
     float* __restrict__ state, long state_stride, const int* __restrict__ q_start, const int* __restrict__ seq_slots,
-    const int* __restrict__ positions, T* __restrict__ out, int parts, int batch, long out_stride, float out_scale) {
+    const int* __restrict__ positions, T* __restrict__ out, int parts, int batch, long out_stride, float out_scale,
+    int input_act, float* __restrict__ raw) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, threads = blockDim.x;
@@ -58,12 +60,14 @@ __global__ __launch_bounds__(1024) void retention_kernel(
       const int t = index / dim, d = index % dim;
       const T* row = projected + static_cast<long>(first + base + t) * stride;
       float qv = to_float(row[q_at + d]), kv = to_float(row[k_at + d]);
+      if (input_act) qv = silu(qv), kv = silu(kv);
       if (d < rot_dims) {
         const int i = d < half ? d : d - half;
         const int pos = min(positions[first + base + t], table_positions - 1);
         const float c = table[(static_cast<long>(pos) * half + i) * 2], s = table[(static_cast<long>(pos) * half + i) * 2 + 1];
         const int other = d < half ? d + half : d - half;
-        const float qo = to_float(row[q_at + other]), ko = to_float(row[k_at + other]);
+        float qo = to_float(row[q_at + other]), ko = to_float(row[k_at + other]);
+        if (input_act) qo = silu(qo), ko = silu(ko);
         qv = d < half ? qv * c - qo * s : qv * c + qo * s;
         kv = d < half ? kv * c - ko * s : kv * c + ko * s;
       }
@@ -72,7 +76,8 @@ __global__ __launch_bounds__(1024) void retention_kernel(
     }
     for (int index = tid; index < tb * vdim; index += threads) {
       const int t = index / vdim, c = index % vdim;
-      vs[index] = to_float(projected[static_cast<long>(first + base + t) * stride + v_at + c]);
+      const float value = to_float(projected[static_cast<long>(first + base + t) * stride + v_at + c]);
+      vs[index] = input_act ? silu(value) : value;
     }
     __syncthreads();
     if (owner) {
@@ -99,10 +104,14 @@ __global__ __launch_bounds__(1024) void retention_kernel(
     }
     __syncthreads();
     for (int t = wave; t < tb; t += waves) {
+      const long n = first + base + t;
+      if (raw != nullptr) {      // the heads' outputs as they are: whoever called norms and gates them
+        for (int c = lane; c < vdim; c += kWave) raw[(n * heads + h) * vdim + c] = os[t * vdim + c];
+        continue;
+      }
       float squares = 0.f;
       for (int c = lane; c < vdim; c += kWave) squares += os[t * vdim + c] * os[t * vdim + c];
       const float scale = rsqrtf(wave_sum(squares) / static_cast<float>(vdim) + eps);
-      const long n = first + base + t;
       for (int c = lane; c < vdim; c += kWave) {
         const float g = to_float(projected[n * stride + g_at + c]);
         out[n * out_stride + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g) * out_scale);
@@ -131,7 +140,7 @@ template <typename T>
 __device__ __forceinline__ void load_chunk(const T* __restrict__ projected, long stride, int heads, int h, int dim, int vdim,
                                            int rot_dims, const float* __restrict__ table, int table_positions,
                                            float key_scale, const int* __restrict__ positions, int first, int n,
-                                           float* qs, float* ks, float* vs, int pitch, bool with_q) {
+                                           float* qs, float* ks, float* vs, int pitch, bool with_q, int input_act) {
   const long q_at = static_cast<long>(h) * dim, k_at = static_cast<long>(heads) * dim + q_at;
   const long v_at = 2L * heads * dim + static_cast<long>(h) * vdim;
   const int half = rot_dims / 2;
@@ -139,30 +148,36 @@ __device__ __forceinline__ void load_chunk(const T* __restrict__ projected, long
     const int t = index / dim, d = index % dim;
     const T* row = projected + static_cast<long>(first + t) * stride;
     float qv = with_q ? to_float(row[q_at + d]) : 0.f, kv = to_float(row[k_at + d]);
+    if (input_act) qv = silu(qv), kv = silu(kv);
     if (d < rot_dims) {
       const int i = d < half ? d : d - half;
       const int pos = min(positions[first + t], table_positions - 1);
       const float c = table[(static_cast<long>(pos) * half + i) * 2], sn = table[(static_cast<long>(pos) * half + i) * 2 + 1];
       const int other = d < half ? d + half : d - half;
-      const float ko = to_float(row[k_at + other]);
+      float ko = to_float(row[k_at + other]);
+      if (input_act) ko = silu(ko);
       kv = d < half ? kv * c - ko * sn : kv * c + ko * sn;
       if (with_q) {
-        const float qo = to_float(row[q_at + other]);
+        float qo = to_float(row[q_at + other]);
+        if (input_act) qo = silu(qo);
         qv = d < half ? qv * c - qo * sn : qv * c + qo * sn;
       }
     }
     if (with_q) qs[t * pitch + d] = qv;
     ks[t * pitch + d] = kv * key_scale;
   }
-  for (int index = threadIdx.x; index < n * vdim; index += blockDim.x)
-    vs[index] = to_float(projected[static_cast<long>(first + index / vdim) * stride + v_at + index % vdim]);
+  for (int index = threadIdx.x; index < n * vdim; index += blockDim.x) {
+    const float value = to_float(projected[static_cast<long>(first + index / vdim) * stride + v_at + index % vdim]);
+    vs[index] = input_act ? silu(value) : value;
+  }
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void retention_chunk_sums_kernel(
     const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
     const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay,
-    const int* __restrict__ q_start, const int* __restrict__ positions, float* __restrict__ sums, int length, int chunks) {
+    const int* __restrict__ q_start, const int* __restrict__ positions, float* __restrict__ sums, int length, int chunks,
+    int input_act) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x, h = blockIdx.y, chunk = blockIdx.z;
   const int first = q_start[seq], count = q_start[seq + 1] - first;
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(256) void retention_chunk_sums_kernel(
   float* vs = ks + length * pitch;   // [length][vdim]
   float* ws = vs + length * vdim;    // [length]
   load_chunk(projected, stride, heads, h, dim, vdim, rot_dims, table, table_positions, key_scale, positions,
-             first + chunk * length, n, nullptr, ks, vs, pitch, false);
+             first + chunk * length, n, nullptr, ks, vs, pitch, false, input_act);
   const float w = decay[h];
   for (int j = threadIdx.x; j < n; j += blockDim.x) ws[j] = power(w, n - 1 - j);
   __syncthreads();
@@ -235,7 +250,7 @@ __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
     const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
     const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay, float eps,
     const int* __restrict__ q_start, const int* __restrict__ positions, const float* __restrict__ states, int length,
-    int chunks, T* __restrict__ out, long out_stride, float out_scale) {
+    int chunks, T* __restrict__ out, long out_stride, float out_scale, int input_act, float* __restrict__ raw) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x, h = blockIdx.y, chunk = blockIdx.z;
   const int first = q_start[seq], count = q_start[seq + 1] - first;
@@ -249,7 +264,7 @@ __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
   float* ws = as + length * (length + 1);   // [length + 1]: w^0 .. w^length
   const int row0 = first + chunk * length;
   load_chunk(projected, stride, heads, h, dim, vdim, rot_dims, table, table_positions, key_scale, positions, row0, n, qs, ks,
-             vs, pitch, true);
+             vs, pitch, true, input_act);
   const float w = decay[h];
   for (int j = threadIdx.x; j <= n; j += blockDim.x) ws[j] = power(w, j);
   __syncthreads();
@@ -304,10 +319,14 @@ __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const long g_at = 2L * heads * dim + static_cast<long>(heads) * vdim + static_cast<long>(h) * vdim;
   for (int t = wave; t < n; t += waves) {
+    const long row = row0 + t;
+    if (raw != nullptr) {
+      for (int c = lane; c < vdim; c += kWave) raw[(row * heads + h) * vdim + c] = os[t * vdim + c];
+      continue;
+    }
     float squares = 0.f;
     for (int c = lane; c < vdim; c += kWave) squares += os[t * vdim + c] * os[t * vdim + c];
     const float scale = rsqrtf(wave_sum(squares) / static_cast<float>(vdim) + eps);
-    const long row = row0 + t;
     for (int c = lane; c < vdim; c += kWave) {
       const float g = to_float(projected[row * stride + g_at + c]);
       out[row * out_stride + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g) * out_scale);
@@ -390,7 +409,7 @@ template <typename T, int GROUPS>
 int launch_retention_outputs(const dim3 grid, size_t lds, hipStream_t stream, const T* projected, long stride, int heads, int dim,
                              int vdim, int rot_dims, const float* table, int table_positions, float key_scale,
                              const float* decay, float eps, const int* q_start, const int* positions, const float* states,
-                             int length, int chunks, T* out, long out_stride, float out_scale) {
+                             int length, int chunks, T* out, long out_stride, float out_scale, int input_act, float* raw) {
   // (asked for once per kernel, for the most a launch may want: a step that is being recorded then changes no attribute)
   static bool allowed = false;
   if (lds > 64 * 1024 && !allowed) {
@@ -402,7 +421,7 @@ int launch_retention_outputs(const dim3 grid, size_t lds, hipStream_t stream, co
   retention_chunk_outputs_kernel<T, GROUPS><<<grid, 256, lds, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
                                                                         table_positions, key_scale, decay, eps, q_start,
                                                                         positions, states, length, chunks, out, out_stride,
-                                                                        out_scale);
+                                                                        out_scale, input_act, raw);
   return 0;
 }
 
@@ -411,7 +430,7 @@ int launch_retention_chunked(const T* projected, long stride, int seqs, int head
                              const float* table, int table_positions, float key_scale, const float* decay, float eps,
                              float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
                              T* out, long out_stride, float out_scale, float* sums, float* states, int length, int chunks,
-                             size_t lds_sums, size_t lds_outputs, hipStream_t stream) {
+                             size_t lds_sums, size_t lds_outputs, int input_act, float* raw, hipStream_t stream) {
   const dim3 grid(seqs, heads, chunks);
   const int size = dim * vdim;
   static bool allowed = false;
@@ -423,13 +442,13 @@ int launch_retention_chunked(const T* projected, long stride, int seqs, int head
   }
   retention_chunk_sums_kernel<T><<<grid, 256, lds_sums, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
                                                                 table_positions, key_scale, decay, q_start, positions, sums,
-                                                                length, chunks);
+                                                                length, chunks, input_act);
   retention_chunk_states_kernel<<<dim3(seqs, heads, (size + 255) / 256), 256, 0, stream>>>(
       sums, states, state, state_stride, decay, q_start, seq_slots, heads, size, length, chunks);
 #define AKV_OUTPUTS(GROUPS)                                                                                               \
   launch_retention_outputs<T, GROUPS>(grid, lds_outputs, stream, projected, stride, heads, dim, vdim, rot_dims, table,       \
                                       table_positions, key_scale, decay, eps, q_start, positions, states, length, chunks, out, \
-                                      out_stride, out_scale)
+                                      out_stride, out_scale, input_act, raw)
   if (vdim <= 32) return AKV_OUTPUTS(8);
   if (vdim <= 64) return AKV_OUTPUTS(4);
   if (vdim <= 128) return AKV_OUTPUTS(2);
@@ -444,7 +463,7 @@ extern "C" {
 int akv_retention(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                   const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
                   long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
-                  long out_stride, float out_scale, hipStream_t stream) {
+                  long out_stride, float out_scale, int input_act, float* raw, hipStream_t stream) {
   if (seqs <= 0) return 0;
   if (heads <= 0 || dim <= 0 || vdim <= 0 || vdim > 1024 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim) return -2;
   if (rot_dims > 0 && (table == nullptr || table_positions <= 0)) return -2;
@@ -467,7 +486,7 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
   AKV_DISPATCH(dtype, T, retention_kernel<T, R><<<grid, threads, lds_of(batch), stream>>>(                             \
                              static_cast<const T*>(projected), stride, heads, dim, vdim, rot_dims, table, table_positions, \
                              key_scale, decay, eps, state, state_stride, q_start, seq_slots, positions,                 \
-                             static_cast<T*>(out), parts, batch, out_stride, out_scale))
+                             static_cast<T*>(out), parts, batch, out_stride, out_scale, input_act, raw))
   switch (per_thread) {
     case 4: AKV_RETENTION(4); break;
     case 8: AKV_RETENTION(8); break;
@@ -484,8 +503,8 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
 int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                           const float* table, int table_positions, float key_scale, const float* decay, float eps,
                           float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
-                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks,
-                          hipStream_t stream) {
+                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks, int input_act,
+                          float* raw, hipStream_t stream) {
   if (seqs <= 0 || chunks <= 0) return 0;
   if (heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || length < 1 || length > 32) return -2;
   if (rot_dims > 0 && (table == nullptr || table_positions <= 0)) return -2;
@@ -498,7 +517,8 @@ int akv_retention_chunked(const void* projected, long stride, int dtype, int seq
   AKV_DISPATCH(dtype, T, status = launch_retention_chunked<T>(
                              static_cast<const T*>(projected), stride, seqs, heads, dim, vdim, rot_dims, table, table_positions,
                              key_scale, decay, eps, state, state_stride, q_start, seq_slots, positions, static_cast<T*>(out),
-                             out_stride, out_scale, sums, states, length, chunks, lds_sums, lds_outputs, stream));
+                             out_stride, out_scale, sums, states, length, chunks, lds_sums, lds_outputs, input_act, raw,
+                             stream));
   if (status != 0) return status;
   return AKV_LAUNCH_STATUS();
 }

@@ -78,7 +78,8 @@ __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restri
                                                                  const float* __restrict__ post_weight, float post_eps,
                                                                  const float* __restrict__ pre_weight, float pre_eps,
                                                                  T* __restrict__ out, int hidden, float delta_scale,
-                                                                 const float* __restrict__ offset) {
+                                                                 const float* __restrict__ offset,
+                                                                 const T* __restrict__ delta2) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float4 kept[GROUPS], added[GROUPS];
@@ -88,6 +89,10 @@ __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restri
     const int i = min((j * 256 + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
     kept[j] = read4<float>(stream + base + i);
     if (delta != nullptr) added[j] = read4<T>(delta + base + i);
+    if (delta2 != nullptr) {      // a second branch beside the first: the two are added in float32 before they meet the sum
+      const float4 b = read4<T>(delta2 + base + i);
+      added[j] = make_float4(added[j].x + b.x, added[j].y + b.y, added[j].z + b.z, added[j].w + b.w);
+    }
   }
   float squares = 0.f;
   if (delta != nullptr) {
@@ -145,7 +150,8 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ 
                                                             const float* __restrict__ post_weight, float post_eps,
                                                             const float* __restrict__ pre_weight, float pre_eps,
                                                             T* __restrict__ out, int hidden, float delta_scale,
-                                                            const float* __restrict__ offset) {
+                                                            const float* __restrict__ offset,
+                                                            const T* __restrict__ delta2) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float* s = stream + base;
@@ -163,8 +169,10 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ 
         }
         post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
       }
-      for (int i = threadIdx.x; i < hidden; i += blockDim.x)
-        s[i] += post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]) * delta_scale;
+      for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float both = delta2 != nullptr ? to_float(d[i]) + to_float(delta2[base + i]) : to_float(d[i]);
+        s[i] += post_weight != nullptr ? both * post_scale * post_weight[i] : both * delta_scale;
+      }
     }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
       const float v = offset != nullptr ? s[i] + offset[i] : s[i];
@@ -210,6 +218,60 @@ __global__ __launch_bounds__(256) void embed_normed_kernel(const int* __restrict
   }
   const float scale = rsqrtf(block_sum(squares, scratch) / static_cast<float>(hidden) + eps);
   for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(row[d]) * scale * weight[d];
+}
+
+// ---- rows of an embedding table into (or onto) the residual sum --------------------------------------------------------
+// out[n] = table[id] (or out[n] += table[id] with `accumulate`), float32; an id of -1 is the token chosen last for the row's
+// request, where the slot words are given.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_rows_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                                         float* __restrict__ out, int hidden, int vocab, int accumulate,
+                                                         const int* __restrict__ seq_of_token,
+                                                         const int* __restrict__ seq_slots,
+                                                         const int* __restrict__ slot_words) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  if (id == -1 && slot_words != nullptr)
+    id = slot_words[static_cast<long>(seq_slots[seq_of_token[n]]) * kSlotWords + kSlotLastToken];
+  float* dst = out + static_cast<size_t>(n) * hidden;
+  if (id < 0 || id >= vocab) {     // never read outside the table; a poisoned row shows the fault downstream
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = __uint_as_float(kPoison);
+    return;
+  }
+  const T* row = table + static_cast<size_t>(id) * hidden;
+  for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = accumulate ? dst[d] + to_float(row[d]) : to_float(row[d]);
+}
+
+// ---- a row's norm, weight and gate in one pass ------------------------------------------------------------------------------
+// x [tokens, width] (TX: float32, or the activation dtype) at `x_stride` per token.  out = x / rms(x) * weight (`normed`; the
+// root mean square over the whole row, `weight` may be null) times act(gate), the gate read from `gates` at `gate_stride`
+// per token (gate_act 0: none, 1: sigmoid, 2: silu), times out_scale.  One block per token; float32 up to the store.
+template <typename TX, typename T>
+__global__ __launch_bounds__(256) void norm_gate_rows_kernel(const TX* __restrict__ x, long x_stride, int width, int normed,
+                                                             const float* __restrict__ weight, float eps,
+                                                             const T* __restrict__ gates, long gate_stride, int gate_act,
+                                                             T* __restrict__ out, long out_stride, float out_scale) {
+  __shared__ float scratch[16];
+  const long n = blockIdx.x;
+  const TX* row = x + n * x_stride;
+  float scale = out_scale;
+  if (normed) {
+    float squares = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float v = to_float(row[i]);
+      squares += v * v;
+    }
+    scale *= rsqrtf(block_sum(squares, scratch) / static_cast<float>(width) + eps);
+  }
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = to_float(row[i]) * scale;
+    if (weight != nullptr) v *= weight[i];
+    if (gate_act != 0) {
+      const float g = to_float(gates[n * gate_stride + i]);
+      v *= gate_act == 1 ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
+    }
+    out[n * out_stride + i] = from_float<T>(v);
+  }
 }
 
 // ---- a gated feed-forward's activation after a stacked product: out = act(gate) * up --------------------------------------
@@ -308,6 +370,34 @@ int akv_difference_norm_gate(const void* maps, const float* lambda, float eps, f
   return AKV_LAUNCH_STATUS();
 }
 
+int akv_embed_rows(const int* ids, const void* table, int dtype, float* out, int tokens, int hidden, int vocab, int accumulate,
+                   const int* seq_of_token, const int* seq_slots, const int* slot_words, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (hidden <= 0 || vocab <= 0) return -2;
+  AKV_DISPATCH(dtype, T, embed_rows_kernel<T><<<tokens, 256, 0, stream>>>(ids, static_cast<const T*>(table), out, hidden, vocab,
+                                                                         accumulate, seq_of_token, seq_slots, slot_words));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_norm_gate_rows(const void* x, int x_dtype, long x_stride, int width, int normed, const float* weight, float eps,
+                       const void* gates, long gate_stride, int gate_act, void* out, int dtype, long out_stride,
+                       float out_scale, long tokens, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (width <= 0 || gate_act < 0 || gate_act > 2 || (gate_act != 0 && gates == nullptr)) return -2;
+  if (x_dtype != kF32 && x_dtype != dtype) return -2;
+  AKV_DISPATCH(dtype, T, {
+    if (x_dtype == kF32 && dtype != kF32)
+      norm_gate_rows_kernel<float, T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
+          static_cast<const float*>(x), x_stride, width, normed, weight, eps, static_cast<const T*>(gates), gate_stride,
+          gate_act, static_cast<T*>(out), out_stride, out_scale);
+    else
+      norm_gate_rows_kernel<T, T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
+          static_cast<const T*>(x), x_stride, width, normed, weight, eps, static_cast<const T*>(gates), gate_stride, gate_act,
+          static_cast<T*>(out), out_stride, out_scale);
+  });
+  return AKV_LAUNCH_STATUS();
+}
+
 int akv_parts_slot_layout(int* out) {
   out[0] = kSlotWords;
   out[1] = kSlotLastToken;
@@ -335,10 +425,11 @@ int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots
 
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      float delta_scale, const float* offset, hipStream_t stream) {
+                      float delta_scale, const float* offset, const void* delta2, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (out != nullptr && pre_weight == nullptr) return -2;
-#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden, delta_scale, offset
+  if (delta2 != nullptr && (delta == nullptr || post_weight != nullptr)) return -2;
+#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden, delta_scale, offset, static_cast<const T*>(delta2)
   AKV_DISPATCH(dtype, T, {
     if (hidden % 4 == 0 && hidden >= 4 && hidden <= 256 * 4 * 2) norm_add_norm_rows_kernel<T, 2><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
     else if (hidden % 4 == 0 && hidden <= 256 * 4 * 8) norm_add_norm_rows_kernel<T, 8><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);

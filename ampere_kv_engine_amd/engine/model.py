@@ -108,6 +108,11 @@ class Model:
             ctx.fold_gain = following.entry_gain() if following is not None and following.takes_stream_sums else None
             if entry.adds_row is not None:
                 pending = self._with_vector(pending, self.pass_vectors.row(entry.adds_row), ctx)
+            if entry.adds_embedding:
+                # (sums commute: the branch that is still to be added meets the residual sum in the next norm's kernel)
+                if isinstance(pending, StreamSums):
+                    raise TypeError("the embedding cannot follow a branch that has left only its rows' sums of squares")
+                self.embedding.add(ctx.token_ids, ctx.stream, ctx)
             if isinstance(pending, Unsettled) and not self.blocks[entry.layer].takes_normed_delta:
                 pending.settle(ctx.stream)       # the reader knows tensors only: the branch is normed and added first
                 pending = None
@@ -138,7 +143,7 @@ class Model:
         times a constant takes the vector along into the kernel that adds it; anything else is settled first."""
         k = self.rt.kernels
         if isinstance(pending, ScaledDelta) and pending.offset is None:
-            return ScaledDelta(pending.delta, pending.scale, k, offset=vector)
+            return ScaledDelta(pending.delta, pending.scale, k, offset=vector, second=pending.second)
         if isinstance(pending, Unsettled):
             pending.settle(ctx.stream)
             pending = None

@@ -47,7 +47,7 @@ class PartsKernels:
                          "akv_parts_slot_layout", "akv_conv_taps", "akv_scaled_sum", "akv_unit_norm_write",
                          "akv_gated_attention_rows", "akv_gated_attention_tiles", "akv_retention", "akv_retention_chunked", "akv_gated_linear_scan", "akv_route_chosen",
                          "akv_gate_silu_mul", "akv_embed_normed", "akv_gated_activation", "akv_difference_norm_gate",
-                         "akv_delta_rule"):
+                         "akv_delta_rule", "akv_embed_rows", "akv_norm_gate_rows", "akv_gate_activation"):
                 getattr(lib, name).restype = ctypes.c_int
             lib.akv_delta_rule_workspace.restype = ctypes.c_long
             layout = (ctypes.c_int * 3)()
@@ -104,16 +104,21 @@ class PartsKernels:
                                             self._stream()), "note_fed_tokens")
 
     def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale: float = 1.0,
-                      offset=None) -> None:
+                      offset=None, delta2=None) -> None:
         """stream (float32) += delta / rms(delta) * post_weight (+= delta_scale * delta where `post_weight` is None; nothing
         where `delta` is None); then stream += offset (a float32 vector, the same on every row) where there is one; then,
-        where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one rounding of a stored result."""
+        where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one rounding of a stored result.
+        `delta2` (beside a `delta` that is not normed): a second branch, stream += delta_scale * (delta + delta2)."""
         tokens, hidden = stream.shape
         self._dense(stream, "stream", torch.float32)
         dtype = None
         if delta is not None:
             self._dense(delta, "delta", None, (tokens, hidden))
             dtype = delta.dtype
+        if delta2 is not None:
+            if delta is None or post_weight is not None:
+                self._refuse("a second branch comes beside a first one that is added as it is")
+            self._dense(delta2, "delta2", delta.dtype, (tokens, hidden))
         if out is not None:
             self._dense(out, "out", dtype, (tokens, hidden))
             self._dense(pre_weight, "pre_weight", torch.float32, (hidden,))
@@ -127,8 +132,65 @@ class PartsKernels:
             return
         self._check(self._parts().akv_norm_add_norm(_ptr(stream), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps),
                                                     _ptr(pre_weight), ctypes.c_float(pre_eps), _ptr(out), _DTYPE_CODE[dtype],
-                                                    tokens, hidden, ctypes.c_float(delta_scale), _ptr(offset), self._stream()),
+                                                    tokens, hidden, ctypes.c_float(delta_scale), _ptr(offset), _ptr(delta2),
+                                                    self._stream()),
                     "norm_add_norm")
+
+    def embed_add(self, ids, table, out, ctx=None) -> None:
+        """out[n] += table[id], float32: the embedding's rows added to a residual sum that already holds something.  With
+        the step's context an id of -1 is the token chosen last for the row's request."""
+        tokens = ids.shape[0]
+        self._dense(ids, "ids", torch.int32, (tokens,))
+        self._dense(table, "table")
+        vocab, hidden = table.shape
+        self._dense(out, "out", torch.float32, (tokens, hidden))
+        words = getattr(ctx, "slot_words", None) if ctx is not None else None
+        seq_of_token = seq_slots = None
+        if words is not None:
+            seq_of_token, seq_slots = ctx.seq_of_token, ctx.seq_slots
+            self._dense(words, "slot_words", torch.int32)
+            self._dense(seq_of_token, "seq_of_token", torch.int32, (tokens,))
+            self._dense(seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+            if max(ctx.host_seq_slots) >= words.shape[0]:
+                self._refuse("a request's slot lies outside the slot words")
+        self._check(self._parts().akv_embed_rows(_ptr(ids), _ptr(table), self._code_of(table), _ptr(out), tokens, hidden, vocab,
+                                                 1, _ptr(seq_of_token), _ptr(seq_slots), _ptr(words), self._stream()),
+                    "embed_add")
+
+    GATE_ACTS = {None: 0, "sigmoid": 1, "silu": 2}
+
+    def norm_gate_rows(self, x, weight, eps, gates, gate_at: int, gate: str | None, out, out_at: int = 0,
+                       out_scale: float = 1.0, x_at: int = 0, width: int | None = None) -> None:
+        """Columns x_at .. x_at + width of `x` (float32, or `out`'s dtype; default: all of them) -> columns out_at .. of
+        `out`: the row divided by its root mean square over all `width` columns (eps inside the root; `eps` None: not
+        normed), times `weight` (float32 [width], may be None), times sigmoid or silu (`gate`) of columns gate_at .. of
+        `gates`, times `out_scale`.  Float32 up to the one rounding."""
+        tokens = x.shape[0]
+        self._dense(x, "x")
+        self._dense(out, "out")
+        if width is None:
+            width = x.shape[1] - x_at
+        if x.dim() != 2 or x_at < 0 or x_at + width > x.shape[1] or width <= 0:
+            self._refuse(f"x must be [tokens, at least {x_at + width}], got {tuple(x.shape)}")
+        if x.dtype != torch.float32 and x.dtype != out.dtype:
+            self._refuse(f"x must be float32 or {out.dtype}, got {x.dtype}")
+        if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + width > out.shape[1]:
+            self._refuse(f"out must be [tokens, at least {out_at + width}], got {tuple(out.shape)}")
+        if weight is not None:
+            self._dense(weight, "weight", torch.float32, (width,))
+        if gate not in self.GATE_ACTS:
+            self._refuse(f"a gate is 'sigmoid', 'silu' or None, not {gate!r}")
+        gate_stride = 0
+        if gate is not None:
+            self._dense(gates, "gates", out.dtype)
+            if gates.dim() != 2 or gates.shape[0] != tokens or gate_at < 0 or gate_at + width > gates.shape[1]:
+                self._refuse(f"gates must be [tokens, at least {gate_at + width}], got {tuple(gates.shape)}")
+            gate_stride = gates.shape[1]
+        self._check(self._parts().akv_norm_gate_rows(
+            _ptr_at(x, x_at), self._code_of(x), _long(x.shape[1]), width, 0 if eps is None else 1, _ptr(weight),
+            ctypes.c_float(eps if eps is not None else 0.0), _ptr_at(gates, gate_at) if gate is not None else ctypes.c_void_p(0),
+            _long(gate_stride), self.GATE_ACTS[gate], _ptr_at(out, out_at), self._code_of(out), _long(out.shape[1]),
+            ctypes.c_float(out_scale), _long(tokens), self._stream()), "norm_gate_rows")
 
     def embed_normed(self, ids, table, weight, eps: float, out, ctx=None) -> None:
         """out[n] = table[id] / rms(table[id]) * weight, float32: an embedding whose rows are normed before the first layer.
@@ -196,13 +258,16 @@ class PartsKernels:
                 and page_size % 8 == 0)
 
     def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
-                      cq, records, latents_t=None) -> None:
+                      cq, records, latents_t=None, interleaved: bool = False) -> None:
         """down [tokens, q_rank (+ kv_rank + rot)] -> cq = norm(q latent); with `records` [pages, 1, page, kv_rank + rot]
         also the token's record: norm(kv latent), then the key part with its first `rot_dims` dimensions rotated; with
-        `latents_t` [pages, 1, kv_rank, page] the normed latent once more, keys contiguous."""
+        `latents_t` [pages, 1, kv_rank, page] the normed latent once more, keys contiguous.  A rotation pair is dimensions
+        (i, i + rot_dims / 2), or (2 i, 2 i + 1) with `interleaved`."""
         tokens = down.shape[0]
         writes = records is not None
-        self._dense(down, "down", None, (tokens, q_rank + (kv_rank + rot if writes else 0)))
+        self._dense(down, "down")
+        if down.dim() != 2 or down.shape[1] < q_rank + (kv_rank + rot if writes else 0):
+            self._refuse(f"down must be [tokens, at least {q_rank + (kv_rank + rot if writes else 0)}], got {tuple(down.shape)}")
         self._dense(cq, "cq", down.dtype, (tokens, q_rank))
         self._dense(q_weight, "q_weight", torch.float32, (q_rank,))
         self._dense(positions, "positions", torch.int32, (tokens,))
@@ -225,9 +290,9 @@ class PartsKernels:
             _ptr(positions), _ptr(slot_map) if writes else ctypes.c_void_p(0), _ptr(cq),
             _ptr(records) if writes else ctypes.c_void_p(0), _long(slots),
             _ptr(latents_t) if writes and latents_t is not None else ctypes.c_void_p(0),
-            records.shape[2] if writes else 0, self._stream()), "latent_encode")
+            records.shape[2] if writes else 0, 1 if interleaved else 0, _long(down.shape[1]), self._stream()), "latent_encode")
 
-    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at) -> None:
+    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at, interleaved: bool = False) -> None:
         """q [tokens, heads * (dim + rot)] -> q_abs[:, :, at:at + rot] (float32, or bfloat16 like q): every head's last
         `rot` dimensions, the first `rot_dims` of them rotated by the token's position."""
         tokens = q.shape[0]
@@ -243,7 +308,8 @@ class PartsKernels:
         self._dense(positions, "positions", torch.int32, (tokens,))
         self._check(self._parts().akv_rotate_queries(_ptr(q), self._code_of(q), _long(tokens), heads, dim, rot, rot_dims,
                                                      _ptr(table), table.shape[0], _ptr(positions), _ptr(q_abs),
-                                                     self._code_of(q_abs), q_abs.shape[2], at, self._stream()),
+                                                     self._code_of(q_abs), q_abs.shape[2], at, 1 if interleaved else 0,
+                                                     self._stream()),
                     "rotate_queries")
 
     def heads_linear(self, x, x_width: int, weight, y, y_width: int) -> None:
@@ -490,14 +556,42 @@ class PartsKernels:
                                                         experts, up.shape[1] // experts, self._stream()),
                     "gate_relu_squared")
 
-    def route_chosen(self, logits, gates, experts: int, top: int) -> None:
+    def route_chosen(self, logits, gates, experts: int, top: int, law: str = "softmax") -> None:
         """gates[t, e] = the softmax over the `top` largest of the first `experts` logits for those experts (equal logits
-        go to the lower index), 0 for the others; every further column of a row becomes its sigmoid."""
-        tokens, scored = logits.shape
+        go to the lower index), 0 for the others; every further column of a row becomes its sigmoid.  `law="sigmoid"`:
+        logits [tokens, experts]; a chosen expert's gate is the sigmoid of its own logit, and every further column of
+        `gates` becomes 1."""
+        tokens = logits.shape[0]
         self._dense(logits, "logits", torch.float32)
-        self._dense(gates, "gates", torch.float32, (tokens, scored))
-        self._check(self._parts().akv_route_chosen(_ptr(logits), _ptr(gates), tokens, experts, scored, top, self._stream()),
-                    "route_chosen")
+        if law == "sigmoid":
+            self._dense(logits, "logits", torch.float32, (tokens, experts))
+            self._dense(gates, "gates", torch.float32)
+            if gates.dim() != 2 or gates.shape[0] != tokens or gates.shape[1] < experts:
+                self._refuse(f"gates must be [tokens, at least {experts}], got {tuple(gates.shape)}")
+        elif law == "softmax":
+            self._dense(gates, "gates", torch.float32, (tokens, logits.shape[1]))
+        else:
+            self._refuse(f"chosen experts are weighted by 'softmax' or 'sigmoid', not {law!r}")
+        self._check(self._parts().akv_route_chosen(_ptr(logits), _ptr(gates), tokens, experts, gates.shape[1], top,
+                                                   1 if law == "sigmoid" else 0, self._stream()), "route_chosen")
+
+    EXPERT_ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu_squared": 3}
+
+    def gate_activation(self, up, gates, act, experts: int, ff: int, activation: str, inside: bool) -> None:
+        """act[t, c] = f(gates[t, e(c)] * up[t, c]) (`inside`) or gates[t, e(c)] * f(up[t, c]); column c belongs to expert
+        c // ff below experts * ff and to the expert every token uses beyond (gate number `experts`); exact zeros where the
+        gate is zero.  (May be in place.)"""
+        tokens, columns = act.shape
+        self._dense(act, "act")
+        self._dense(up, "up", act.dtype, (tokens, columns))
+        self._dense(gates, "gates", torch.float32)
+        if gates.dim() != 2 or gates.shape[0] != tokens or gates.shape[1] < experts + (1 if columns > experts * ff else 0):
+            self._refuse(f"gates must be [tokens, at least the experts (and the shared one)], got {tuple(gates.shape)}")
+        if activation not in self.EXPERT_ACTIVATIONS:
+            self._refuse(f"an expert's activation is one of {sorted(self.EXPERT_ACTIVATIONS)}, not {activation!r}")
+        self._check(self._parts().akv_gate_activation(_ptr(up), _ptr(gates), _ptr(act), self._code_of(act), _long(tokens),
+                                                      experts, ff, columns, gates.shape[1], self.EXPERT_ACTIVATIONS[activation],
+                                                      1 if inside else 0, self._stream()), "gate_activation")
 
     def gate_silu_mul(self, gate_up, gates, act, experts: int, ff: int) -> None:
         """act[t, c] = gates[t, e(c)] * silu(gate_up[t, c]) * gate_up[t, columns + c]; column c belongs to expert c // ff
@@ -529,14 +623,21 @@ class PartsKernels:
         return k_pages.shape[0], k_pages.shape[2]
 
     def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at: int = 0,
-                        maps: int = 1, table=None, rot_dims: int = 0, positions=None) -> None:
+                        maps: int = 1, table=None, rot_dims: int = 0, positions=None, q_weight=None, k_weight=None,
+                        whole: bool = False, interleaved: bool = False) -> None:
         """projected [tokens, ... | q | k | v | ...] with q at column `at`: the query heads divided by their root mean square (eps inside the root;
         `eps` None: as they are) -> q_out; with `slot_map` the key heads, the same way, and the value heads into the
         tokens' slots of the pages.  `maps` > 1: a head's queries and keys are `maps` vectors of `dim` side by side, each
         normed and rotated for itself; a key head's record in the pages is `maps * dim` wide.  `table` [positions,
         rot_dims / 2, 2] (cos, sin): every vector's first `rot_dims` dimensions are rotated by the token's position
-        (`positions`), dimension i with i + rot_dims / 2, after the norm."""
+        (`positions`), dimension i with i + rot_dims / 2 (`interleaved`: 2 i with 2 i + 1), after the norm.  `whole`: the
+        root mean square is taken over all of a token's query vectors at once, and over all its key vectors.  `q_weight`,
+        `k_weight` (float32, one value per column of the queries and of the keys): multiplied in after the norm."""
         tokens = projected.shape[0]
+        if q_weight is not None:
+            self._dense(q_weight, "q_weight", torch.float32, (q_heads * maps * dim,))
+        if k_weight is not None:
+            self._dense(k_weight, "k_weight", torch.float32, (kv_heads * maps * dim,))
         self._dense(projected, "projected")
         if projected.dim() != 2 or at < 0 or projected.shape[1] < at + (q_heads + kv_heads) * maps * dim + kv_heads * vdim:
             self._refuse(f"projected rows must hold queries, keys and values, got {tuple(projected.shape)}")
@@ -557,17 +658,18 @@ class PartsKernels:
             vdim, ctypes.c_float(eps if eps is not None else 0.0), 0 if eps is None else 1, _ptr(slot_map), _ptr(k_pages),
             _ptr(v_pages), page_size, _long(num_pages), _ptr(q_out), maps, _ptr(table), table_positions,
             rot_dims if table is not None else 0, _ptr(positions) if table is not None else ctypes.c_void_p(0),
-            self._stream()), "unit_norm_write")
+            _ptr(q_weight), _ptr(k_weight), 1 if whole else 0, 1 if interleaved else 0, self._stream()), "unit_norm_write")
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
                         chunk, window, sink, out, out_at: int = 0, out_scale: float = 1.0, sink_logits=None,
-                        maps: int = 1) -> None:
+                        maps: int = 1, keep_first: int = 0) -> None:
         """Every query head attends the keys of its request that it sees (see `parts/gated_attention.py`) -> columns
         out_at .. out_at + q_heads * vdim of `out`, times `out_scale`; `gates` [tokens, width]: head h's output times
         sigmoid(gates[t, gate_at + h]).  `sink_logits` [q_heads] float32 (with `sink`): the denominator's extra term is
         exp(sink_logits[h]) instead of exp(0).  `maps` > 1: a head has `maps` query vectors, each an attention of its own
         over the vector of the same number in its key head's record ([pages, kv_heads, page, maps * dim]) and over the
-        head's values; out then holds q_heads * maps outputs a token, a head's maps side by side."""
+        head's values; out then holds q_heads * maps outputs a token, a head's maps side by side.  `keep_first`: a request's
+        first so many keys stay visible behind the window."""
         tokens = q.shape[0]
         heads = q_heads
         q_heads = heads * maps          # (from here on: query vectors)
@@ -602,7 +704,7 @@ class PartsKernels:
             self._refuse("a request is longer than its row of the block table")
         tail = (ctypes.c_float(scale), ctypes.c_float(softcap if softcap is not None else 0.0),
                 int(chunk) if chunk is not None else 0, int(window) if window is not None else 0, 1 if sink else 0,
-                _long(out.shape[1]), ctypes.c_float(out_scale), _ptr(sink_logits), maps, self._stream())
+                _long(out.shape[1]), ctypes.c_float(out_scale), _ptr(sink_logits), maps, int(keep_first), self._stream())
         singles = tokens
         if (q.dtype == torch.bfloat16 and dim in self.MATRIX_CORE_HEAD_DIMS and vdim in self.MATRIX_CORE_HEAD_DIMS
                 and page_size % 16 == 0 and out.shape[1] % 4 == 0 and out_at % 4 == 0):
@@ -621,8 +723,8 @@ class PartsKernels:
             self._check(self._parts().akv_gated_attention_rows(
                 _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
                 _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr_at(out, out_at),
-                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail[:-3], row_waves,
-                *tail[-3:]), "gated_attention")
+                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail[:-4], row_waves,
+                *tail[-4:]), "gated_attention")
 
     # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
     def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:
@@ -630,17 +732,27 @@ class PartsKernels:
             self._refuse(f"retention keeps a head's state [{dim}, {vdim}] in one block's registers: up to 65,536 values")
 
     def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out, at: int = 0,
-                  out_at: int = 0, out_scale: float = 1.0) -> None:
+                  out_at: int = 0, out_scale: float = 1.0, input_activation: str | None = None, raw=None) -> None:
         """projected [tokens, ... | q | k | v | g | ...] with q at column `at` -> columns out_at .. out_at + heads * vdim of
         `out` = (S^T q) / rms * silu(g) * out_scale with S <- decay S + k v^T per request and head (see
-        `parts/retention.py`); S lies in the request's slot of `state`, float32."""
+        `parts/retention.py`); S lies in the request's slot of `state`, float32.  `input_activation="silu"`: q, k and v
+        pass silu as they are read.  `raw` [tokens, heads * vdim] float32: the outputs S^T q are left there as they are,
+        `out` (then None) is not written, and the rows need hold no gates."""
         tokens = projected.shape[0]
         self._dense(projected, "projected")
-        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + 2 * heads * (dim + vdim):
+        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + heads * (2 * dim + vdim) + (heads * vdim if raw is None else 0):
             self._refuse(f"projected rows must hold queries, keys, values and gates from column {at}, got {tuple(projected.shape)}")
-        self._dense(out, "out", projected.dtype)
-        if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + heads * vdim > out.shape[1]:
-            self._refuse(f"out must be [tokens, at least {out_at + heads * vdim}], got {tuple(out.shape)}")
+        if input_activation not in (None, "silu"):
+            self._refuse(f"retention's inputs pass 'silu' or nothing, not {input_activation!r}")
+        if raw is not None:
+            self._dense(raw, "raw", torch.float32, (tokens, heads * vdim))
+            if out is not None:
+                self._refuse("raw outputs are left instead of normed and gated ones")
+            out, out_at = raw, 0      # (stands in where an address is formed; the kernels do not write it)
+        else:
+            self._dense(out, "out", projected.dtype)
+            if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + heads * vdim > out.shape[1]:
+                self._refuse(f"out must be [tokens, at least {out_at + heads * vdim}], got {tuple(out.shape)}")
         self._dense(decay, "decay", torch.float32, (heads,))
         self._dense(state, "state", torch.float32)
         if state.dim() != 2 or state.shape[1] != heads * dim * vdim:
@@ -658,15 +770,16 @@ class PartsKernels:
                 rot_dims, _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
                 ctypes.c_float(eps), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
                 _ptr(ctx.positions), _ptr_at(out, out_at), _long(out.shape[1]), ctypes.c_float(out_scale))
+        extras = (1 if input_activation == "silu" else 0, _ptr(raw))
         length = self._retention_chunk(dim, vdim)
         if ctx.max_new_tokens >= self.RETENTION_CHUNKED_FROM and length:
             # portions: chunks side by side (the step's shape alone decides, so a recorded step replays the same launches)
             chunks = (ctx.max_new_tokens + length - 1) // length
             sums = self._retention_sums(2 * ctx.num_seqs * heads * chunks * dim * vdim)
-            self._check(self._parts().akv_retention_chunked(*head, _ptr(sums), length, chunks, self._stream()),
+            self._check(self._parts().akv_retention_chunked(*head, _ptr(sums), length, chunks, *extras, self._stream()),
                         "retention over chunks")
             return
-        self._check(self._parts().akv_retention(*head, self._stream()), "retention")
+        self._check(self._parts().akv_retention(*head, *extras, self._stream()), "retention")
 
     RETENTION_CHUNKED_FROM = 24       # steps whose longest portion has fewer tokens take them one after the other
 

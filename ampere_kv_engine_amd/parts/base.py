@@ -94,6 +94,7 @@ class PagedKV:
     value_dim: int | None = None
     chunk: int | None = None        # queries see keys of their own chunk of so many positions only (counted from 0):
                                     # the pages of chunks that have been left are given back while the request lives
+    keep_first: int = 0             # a request's first so many tokens stay visible behind the window: their pages are kept
 
     @property
     def v_dim(self) -> int:
@@ -244,13 +245,17 @@ class Unsettled:
 class ScaledDelta(Unsettled):
     """A branch's output that is added to the residual sum times a constant: stream += scale * delta - and then, where
     the model's pass has given one, a vector `offset` that every row takes (what a pass over repeated layers adds before
-    its first layer).  `delta` None: the offset alone."""
+    its first layer).  `delta` None: the offset alone.  `second`: the output of a second branch that read the same
+    input - stream += scale * (delta + second), the two added in float32."""
 
-    def __init__(self, delta: torch.Tensor | None, scale: float, kernels, offset: torch.Tensor | None = None):
-        self.delta, self.scale, self.kernels, self.offset = delta, float(scale), kernels, offset
+    def __init__(self, delta: torch.Tensor | None, scale: float, kernels, offset: torch.Tensor | None = None,
+                 second: torch.Tensor | None = None):
+        self.delta, self.scale, self.kernels, self.offset, self.second = delta, float(scale), kernels, offset, second
 
     def settle(self, stream: torch.Tensor) -> None:
-        self.kernels.norm_add_norm(stream, self.delta, None, 0.0, None, 0.0, None, delta_scale=self.scale, offset=self.offset)
+        more = {"delta2": self.second} if self.second is not None else {}
+        self.kernels.norm_add_norm(stream, self.delta, None, 0.0, None, 0.0, None, delta_scale=self.scale, offset=self.offset,
+                                   **more)
 
 
 class NormedDelta(Unsettled):

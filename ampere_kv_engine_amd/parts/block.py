@@ -195,6 +195,45 @@ class ScaledPreNormBlock(Part):
         return ScaledDelta(self.feed_forward.forward(normed, ctx), self.scale, self.rt.kernels)
 
 
+class SharedNormBlock(Part):
+    """One norm, and both branches read its output:
+        n = norm(h);  h' = h + m * (mixer(n) + feed_forward(n))
+    (a layer without a feed-forward adds the mixer alone).  The norm is float32 up to its one rounding; the two outputs
+    travel on together as one `ScaledDelta` and are added - to each other in float32, then to the residual sum - inside
+    the kernel of the next block's norm, or at the model's end."""
+    graph_safe = True
+    takes_normed_delta = True
+
+    def __init__(self, spec, runtime, mixer, feed_forward):
+        self.rt = runtime
+        self.hidden = int(spec["hidden_size"])
+        self.scale = float(spec.get("residual_scale", 1.0))
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.has_feed_forward = not isinstance(feed_forward, NoFeedForward)
+        self.name = spec.get("name", "norm1")
+        self.norm = build_part("norm", spec["norm"], runtime)
+
+    def tensors(self, prefix):
+        return self.norm.tensors(prefix + self.name) + self.mixer.tensors(prefix) + self.feed_forward.tensors(prefix)
+
+    def load(self, fetch, prefix):
+        self.norm.load(fetch, prefix + self.name)
+        self.mixer.load(fetch, prefix)
+        self.feed_forward.load(fetch, prefix)
+
+    def weight_bytes(self):
+        return self.mixer.weight_bytes() + self.feed_forward.weight_bytes() + self.norm.weight_bytes()
+
+    def forward(self, stream, pending, ctx, cache, writes_cache=True):
+        if pending is not None and not isinstance(pending, Unsettled):
+            raise TypeError("a block with one norm is handed a branch that is still to be added, or nothing")
+        ctx.fold_into_stream, ctx.fold_gain = False, None      # no branch of this block adds itself to the stream
+        normed = self.norm.after(stream, pending, ctx.arena.take((stream.shape[0], self.hidden), self.rt.dtype))
+        mixed = self.mixer.forward(normed, ctx, cache, writes_cache)
+        other = self.feed_forward.forward(normed, ctx) if self.has_feed_forward else None
+        return ScaledDelta(mixed, self.scale, self.rt.kernels, second=other)
+
+
 class NoFeedForward(Part):
     """The feed-forward of a layer that has none."""
     graph_safe = True
@@ -207,4 +246,6 @@ register_part("block", "sandwich", lambda spec, runtime, mixer=None, feed_forwar
               SandwichBlock(spec, runtime, mixer, feed_forward))
 register_part("block", "scaled_prenorm", lambda spec, runtime, mixer=None, feed_forward=None:
               ScaledPreNormBlock(spec, runtime, mixer, feed_forward))
+register_part("block", "shared_norm", lambda spec, runtime, mixer=None, feed_forward=None:
+              SharedNormBlock(spec, runtime, mixer, feed_forward))
 register_part("feed_forward", "none", NoFeedForward)

@@ -32,6 +32,13 @@ class Embedding(Part):
         self.rt.kernels.embed(token_ids, self.weight, stream, ctx)
         return stream
 
+    def add(self, token_ids: torch.Tensor, stream: torch.Tensor, ctx=None) -> None:
+        """stream += the tokens' rows once more: what a pass over repeated layers adds before its first layer where the
+        run order says so (`RunEntry.adds_embedding`).  The rows are gathered again rather than kept."""
+        if type(self) is not Embedding:
+            raise NotImplementedError("only the plain embedding's output is added to the residual sum a second time")
+        self.rt.kernels.embed_add(token_ids, self.weight, stream, ctx)
+
 
 class NormedEmbedding(Embedding):
     """The token's row, normed before the first layer: x = norm(table[id]), in float32 (one kernel).  `norm` is the

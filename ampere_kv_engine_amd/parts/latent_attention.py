@@ -11,6 +11,10 @@ so nothing but the records is ever read from the cache, for prompts and single t
 j with 0 <= i - j < window.  A layer may have no down-projection of its own and read another layer's records
 (`own_latent = False`, with the run order naming that layer's cache); the pages are then kept for the widest window
 among the readers (`cache_window`).  Norms, angles, scores, softmax weights and the weighted sums are float32.
+Without a window every earlier key is seen.  `position` (a `rope_scaled` specification) replaces the plain rotation of
+`rotary_base`: stretched frequencies, a factor on cos and sin, pairs in halves or interleaved.  With `gate` the heads'
+outputs are multiplied, value by value, with sigmoid(W_g h) before the output product (tensor `g`, stacked with the
+down-projections: it reads the same input).
 """
 
 from __future__ import annotations
@@ -48,11 +52,21 @@ class LatentAttention(Part):
         if self.own_latent:
             down_outs.append(self.record)
             down_names.append("dkv")
+        self.gate = bool(spec.get("gate", False))
+        if self.gate:
+            down_outs.append(self.heads * self.vdim)
+            down_names.append("g")
         self.down = Linear(runtime, self.hidden, down_outs, down_names)
         self.up_q = Linear(runtime, self.q_rank, [self.heads * (self.dim + self.rot)], ["uq"])
         self.out = Linear(runtime, self.heads * self.vdim, [self.hidden], ["o"])
-        self.position = build_part("position", part("rope_half", head_dim=self.rot_dims, theta=float(spec["rotary_base"])),
-                                   runtime)
+        if spec.get("position") is not None:
+            self.position = build_part("position", spec["position"], runtime)
+            if self.position.dims != self.rot_dims:
+                raise ValueError(f"the rotation turns {self.position.dims} dimensions, the layer says {self.rot_dims}")
+        else:
+            self.position = build_part("position", part("rope_half", head_dim=self.rot_dims, theta=float(spec["rotary_base"])),
+                                       runtime)
+        self.interleaved = bool(getattr(self.position, "interleaved", False))
         # where the kernel set has a matrix-core kernel for these sizes the layer keeps the latents twice: inside the
         # records, and once more with the keys contiguous, as that kernel's second product reads them
         # (the copy is kept by the layer that writes the records, for whichever of their readers has such a kernel:
@@ -120,20 +134,28 @@ class LatentAttention(Part):
         turned = cache.v if self.on_matrix_cores else None
         k.latent_encode(down, self.q_rank, self.kv_rank, self.rot, self.rot_dims, self.q_norm_weight, self.kv_norm_weight,
                         self.eps, self.position.table, ctx.positions, meta.slot_map, cq, cache.k if writes_cache else None,
-                        latents_t=cache.v if writes_cache else None)
+                        latents_t=cache.v if writes_cache else None, **self._pairs())
         q = ctx.arena.take((tokens, self.heads * (self.dim + self.rot)), dtype)
         self.up_q.forward(cq, q)
         between = dtype if turned is not None else torch.float32      # the matrix cores take their queries in bfloat16
         q_abs = ctx.arena.take((tokens, self.heads, self.record), between)
         k.heads_linear(q.view(tokens, self.heads, self.dim + self.rot), self.dim + self.rot, self.key_up, q_abs, self.record)
         k.rotate_queries(q, self.heads, self.dim, self.rot, self.rot_dims, self.position.table, ctx.positions, q_abs,
-                         self.kv_rank)
+                         self.kv_rank, **self._pairs())
         mixed = ctx.arena.take((tokens, self.heads, self.kv_rank), between)
         k.latent_attend(q_abs, cache.k, ctx, meta, self.heads, self.kv_rank, self.scale, self.window, mixed, latents_t=turned)
         values = ctx.arena.take((tokens, self.heads, self.vdim), dtype)
         k.heads_linear(mixed, self.kv_rank, self.value_up, values, self.vdim)
+        values = values.view(tokens, self.heads * self.vdim)
+        if self.gate:
+            gated = ctx.arena.take((tokens, self.heads * self.vdim), dtype)
+            k.norm_gate_rows(values, None, None, down, self.down.total_out - self.heads * self.vdim, "sigmoid", gated)
+            values = gated
         out = ctx.arena.take((tokens, self.hidden), dtype)
-        return self.out.forward(values.view(tokens, self.heads * self.vdim), out)
+        return self.out.forward(values, out)
+
+    def _pairs(self):
+        return {"interleaved": True} if self.interleaved else {}
 
 
 register_part("mixer", "latent_attention", LatentAttention)

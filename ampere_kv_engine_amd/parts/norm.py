@@ -8,7 +8,8 @@ the folding of norms into products; it can be added to the residual sum as it is
 with the norm that follows (`after`): the norm kernel of blocks that norm a branch before and after.
 
 With `unit_offset` the file stores the weight around zero and the norm multiplies by 1 + w; the sum is formed once, at
-load, in float32."""
+load, in float32.  With `output_scale` the normed rows are multiplied by a constant as well (a model whose logits are
+its head's product times a constant puts it on its final norm): the weight takes it once, at load, in float32."""
 
 from __future__ import annotations
 
@@ -29,6 +30,7 @@ class RMSNorm(Norm):
         self.eps = float(spec["eps"])
         self.single_rounding = bool(spec.get("single_rounding", False))
         self.unit_offset = bool(spec.get("unit_offset", False))
+        self.output_scale = float(spec.get("output_scale", 1.0))
         self.rt = runtime
         self.weight: torch.Tensor | None = None
 
@@ -43,6 +45,8 @@ class RMSNorm(Norm):
         self.weight = fetch(TensorSpec(name, (self.size,), self.role)).to(torch.float32).contiguous()
         if self.unit_offset:
             self.weight += 1.0
+        if self.output_scale != 1.0:
+            self.weight *= self.output_scale
 
     def weight_bytes(self):
         return self.size * 4
@@ -73,8 +77,9 @@ class RMSNorm(Norm):
 
     def after(self, stream, pending, out):
         if isinstance(pending, ScaledDelta) and self.single_rounding:      # one kernel: add the branch times its constant, norm
+            more = {"delta2": pending.second} if pending.second is not None else {}
             self.rt.kernels.norm_add_norm(stream, pending.delta, None, 0.0, self.weight, self.eps, out,
-                                          delta_scale=pending.scale, offset=pending.offset)
+                                          delta_scale=pending.scale, offset=pending.offset, **more)
             return out
         if (pending is None or not isinstance(pending, NormedDelta)
                 or not (self.single_rounding and type(pending.norm) is RMSNorm and pending.norm.single_rounding)):

@@ -10,6 +10,8 @@ f_i = base^(-2i / dims) that a rule stretches for contexts longer than the `orig
   * "llama3": with the wavelength l_i = 2 pi / f_i: f_i stays where l_i < original / high, becomes f_i / factor where
     l_i > original / low, and between the two, with s = (original / l_i - low) / (high - low), (1 - s) f_i / factor + s f_i;
   * none: the frequencies as they are.
+`layout` says which dimensions pair i turns: "halves" (i with i + dims / 2, the default) or "interleaved" (2 i with 2 i + 1);
+the table is the same, the mixer's kernels are told.
 Frequencies are formed in double precision and rounded once; angles are float32 products of position and frequency."""
 
 from __future__ import annotations
@@ -82,6 +84,10 @@ class ScaledRotary(Part):
     def __init__(self, spec, runtime):
         self.rt = runtime
         self.dims, self.base = int(spec["dims"]), float(spec["base"])
+        self.layout = spec.get("layout", "halves")
+        if self.layout not in ("halves", "interleaved"):
+            raise ValueError(f"a rotation pairs dimensions in 'halves' or 'interleaved', not {self.layout!r}")
+        self.interleaved = self.layout == "interleaved"
         scaling = spec.get("scaling")
         if self.dims <= 0 or self.dims % 2:
             raise ValueError(f"a rotation turns an even number of dimensions, got {self.dims}")

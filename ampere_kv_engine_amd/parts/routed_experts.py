@@ -6,11 +6,16 @@ Two laws of choosing and weighting (`weights`):
                       be chosen; the `top` best of those are, weighted by their own scores as they are.
     "softmax_chosen"  logits = W_r h (+ b_r); the `top` experts with the largest logits are chosen and weighted by the
                       softmax over their logits alone.
-Two forms of an expert (`activation`), none with biases:
+    "sigmoid_chosen"  scores = sigmoid(W_r h); the `top` experts with the largest scores are chosen and weighted by their
+                      own scores as they are.
+Forms of an expert (`activation`), none with biases:
     "relu_squared"    W_down relu(W_up h)^2
     "silu_gated"      W_down (silu(W_gate h) * (W_up h))
-and, with `shared_size`, one more expert of that width which every token uses, weighted by sigmoid(w_sg . h), one number a
-token - added to the chosen experts' weighted sum.
+    "gelu"            W_down gelu(W_up h), the exact (erf) gelu
+With `weight_on_input` the router's weight multiplies what the expert reads, not what it returns: expert(w h) - for an
+expert without biases that is the activation of w (W_up h).
+With `shared_size`, one more expert of that width which every token uses, added to the chosen experts' weighted sum -
+weighted by sigmoid(w_sg . h), one number a token (`shared_gate`, the default), or as it is.
 
 The experts' first matrices are stacked into one [experts * ff (+ shared), hidden] (gates, then ups, where an expert
 has both) and their second ones side by side into one [hidden, experts * ff (+ shared)]: a step is the router (the
@@ -28,8 +33,8 @@ from ..weights.spec import MATRIX, TensorSpec
 from .base import Part, register_part
 from .linear import Linear
 
-ACTIVATIONS = ("relu_squared", "silu_gated")
-WEIGHTS = ("softmax_all", "softmax_chosen")
+ACTIVATIONS = ("relu_squared", "silu_gated", "gelu")
+WEIGHTS = ("softmax_all", "softmax_chosen", "sigmoid_chosen")
 
 
 class RoutedExperts(Part):
@@ -52,10 +57,16 @@ class RoutedExperts(Part):
             raise ValueError(f"{self.experts} experts do not form {self.groups} equal groups of which {self.kept} are kept")
         if not 0 < self.top <= self.kept * (self.experts // self.groups):
             raise ValueError(f"{self.top} experts a token cannot be chosen from {self.kept} groups of {self.experts // self.groups}")
-        if self.weights == "softmax_chosen" and self.groups != 1:
-            raise ValueError("the softmax over the chosen experts' logits knows no groups")
-        if self.shared and (self.weights != "softmax_chosen" or self.activation != "silu_gated"):
-            raise ValueError("a shared expert comes with gated experts that are weighted by the softmax over the chosen")
+        if self.weights != "softmax_all" and self.groups != 1:
+            raise ValueError("weights over the chosen experts alone know no groups")
+        self.inside = bool(spec.get("weight_on_input", False))
+        self.shared_gate = bool(spec.get("shared_gate", True)) and bool(self.shared)
+        # which kernels take the step: the gated pair of Tukevik's experts, or one activation with the weight in or outside
+        self.plain = self.activation == "gelu" or self.inside or self.weights == "sigmoid_chosen"
+        if self.plain and (self.activation == "silu_gated" or self.weights != "sigmoid_chosen" or self.shared_gate):
+            raise ValueError("experts weighted by their sigmoid scores are ungated, and so is the expert they share")
+        if not self.plain and self.shared and (self.weights != "softmax_chosen" or self.activation != "silu_gated"):
+            raise ValueError("a shared expert behind a gate comes with gated experts weighted by the softmax over the chosen")
         self.gated = self.activation == "silu_gated"
         first = [f"e{e}.up" for e in range(self.experts)] + (["shared.up"] if self.shared else [])
         sizes = [self.ff] * self.experts + ([self.shared] if self.shared else [])
@@ -68,7 +79,7 @@ class RoutedExperts(Part):
         # the router's logits are a product like any other, with float32 sums left as they are: what the file stores in
         # 16 bits is exact in the operands, so nothing of the logits is formed in less than 32 bits
         bias = "router.b" if spec.get("router_bias", False) else None
-        if self.shared:
+        if self.shared_gate:
             self.router = Linear(runtime, self.hidden, [self.experts, 1], ["router", "shared.sg"],
                                  bias_names=[bias, None] if bias else None)
         else:
@@ -100,6 +111,16 @@ class RoutedExperts(Part):
         k, dtype = self.rt.kernels, self.rt.dtype
         tokens = x.shape[0]
         scored = self.experts + (1 if self.shared else 0)
+        if self.plain:
+            logits = ctx.arena.take((tokens, self.experts), torch.float32)
+            self.router.forward(x, logits)
+            gates = ctx.arena.take((tokens, scored), torch.float32)
+            k.route_chosen(logits, gates, self.experts, self.top, law="sigmoid")      # (the shared expert's gate is 1)
+            up = ctx.arena.take((tokens, self.columns), dtype)
+            self.up.forward(x, up)
+            act = ctx.arena.take((tokens, self.columns), dtype)
+            k.gate_activation(up, gates, act, self.experts, self.ff, self.activation, self.inside)
+            return self.down.forward(act, ctx.arena.take((tokens, self.hidden), dtype))
         logits = ctx.arena.take((tokens, scored), torch.float32)
         self.router.forward(x, logits)
         gates = ctx.arena.take((tokens, scored), torch.float32)

@@ -267,9 +267,10 @@ class TorchKernels(KernelSet):
         out.copy_(table[cur].float() + pairs[rows].float())
         words[ctx.seq_slots.long(), 7] = cur[ctx.q_start.long()[1:] - 1].int()
 
-    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale=1.0, offset=None):
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale=1.0, offset=None,
+                      delta2=None):
         if delta is not None:
-            d = delta.float() * delta_scale
+            d = (delta.float() + delta2.float() if delta2 is not None else delta.float()) * delta_scale
             if post_weight is not None:
                 d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight
             stream += d
@@ -277,6 +278,24 @@ class TorchKernels(KernelSet):
             stream += offset
         if out is not None:
             out.copy_((stream * torch.rsqrt((stream * stream).mean(-1, keepdim=True) + pre_eps) * pre_weight).to(out.dtype))
+
+    def embed_add(self, ids, table, out, ctx=None):
+        """out[n] += table[id]; an id of -1 is the token chosen last for the row's request."""
+        rows = torch.empty_like(out)
+        self.embed(ids, table, rows, ctx)
+        out += rows
+
+    def norm_gate_rows(self, x, weight, eps, gates, gate_at, gate, out, out_at=0, out_scale=1.0, x_at=0, width=None):
+        width = x.shape[1] - x_at if width is None else width
+        v = x[:, x_at:x_at + width].float()
+        if eps is not None:
+            v = v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps)
+        if weight is not None:
+            v = v * weight
+        if gate is not None:
+            g = gates[:, gate_at:gate_at + width].float()
+            v = v * (torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g))
+        out[:, out_at:out_at + width] = (v * out_scale).to(out.dtype)
 
     def embed_normed(self, ids, table, weight, eps, out, ctx=None):
         """out[n] = table[id] / rms(table[id]) * weight; an id of -1 is the token chosen last for the row's request."""
@@ -331,16 +350,21 @@ class TorchKernels(KernelSet):
             state[slot, :heads * dim * vdim] = S.transpose(1, 2).reshape(-1)
 
     @staticmethod
-    def _turn(x, positions, table, rot_dims):
-        """x [..., tokens, heads, rot] float: the first rot_dims dimensions rotated in halves by the table's angles."""
+    def _turn(x, positions, table, rot_dims, interleaved=False):
+        """x [..., tokens, heads, rot] float: the first rot_dims dimensions rotated by the table's angles, pair i being
+        dimensions (i, i + rot_dims / 2) - or (2 i, 2 i + 1) where the pairs are interleaved."""
         half = rot_dims // 2
         cos = table[positions.long(), :, 0][:, None, :]
         sin = table[positions.long(), :, 1][:, None, :]
+        if interleaved:
+            u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+            turned = torch.stack((u * cos - v * sin, v * cos + u * sin), dim=-1).flatten(-2)
+            return torch.cat((turned, x[..., rot_dims:]), dim=-1)
         u, v = x[..., :half], x[..., half:rot_dims]
         return torch.cat((u * cos - v * sin, v * cos + u * sin, x[..., rot_dims:]), dim=-1)
 
     def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
-                      cq, records, latents_t=None):
+                      cq, records, latents_t=None, interleaved=False):
         d = down.float()
         ql = d[:, :q_rank]
         cq.copy_((ql * torch.rsqrt((ql * ql).mean(-1, keepdim=True) + eps) * q_weight).to(cq.dtype))
@@ -348,13 +372,13 @@ class TorchKernels(KernelSet):
             return
         c = d[:, q_rank:q_rank + kv_rank]
         c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * kv_weight
-        key = self._turn(d[:, None, q_rank + kv_rank:], positions, table, rot_dims)[:, 0]
+        key = self._turn(d[:, None, q_rank + kv_rank:q_rank + kv_rank + rot], positions, table, rot_dims, interleaved)[:, 0]
         flat = records.view(-1, kv_rank + rot)
         flat[slot_map.long()] = torch.cat((c, key), dim=-1).to(records.dtype)
 
-    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at):
+    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at, interleaved=False):
         part = q.float().view(q.shape[0], heads, dim + rot)[..., dim:]
-        q_abs[..., at:at + rot] = self._turn(part, positions, table, rot_dims)
+        q_abs[..., at:at + rot] = self._turn(part, positions, table, rot_dims, interleaved)
 
     def heads_linear(self, x, x_width, weight, y, y_width):
         heads, ins, outs = weight.shape
@@ -431,7 +455,7 @@ class TorchKernels(KernelSet):
         pass
 
     def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at=0, maps=1,
-                        table=None, rot_dims=0, positions=None):
+                        table=None, rot_dims=0, positions=None, q_weight=None, k_weight=None, whole=False, interleaved=False):
         projected = projected[:, at:]
         n = projected.shape[0]
         q_size, k_size, v_size = q_heads * maps * dim, kv_heads * maps * dim, kv_heads * vdim
@@ -439,10 +463,15 @@ class TorchKernels(KernelSet):
         k = projected[:, q_size:q_size + k_size].reshape(n, kv_heads * maps, dim).float()
         v = projected[:, q_size + k_size:q_size + k_size + v_size].reshape(n, kv_heads, vdim)
         if eps is not None:
-            q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)
-            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)
+            over = (-2, -1) if whole else -1        # (`whole`: one root mean square for all of a token's query vectors)
+            q = q * torch.rsqrt((q * q).mean(over, keepdim=True) + eps)
+            k = k * torch.rsqrt((k * k).mean(over, keepdim=True) + eps)
+        if q_weight is not None:
+            q = q * q_weight.view(q_heads * maps, dim)
+        if k_weight is not None:
+            k = k * k_weight.view(kv_heads * maps, dim)
         if table is not None:
-            q, k = self._turn(q, positions, table, rot_dims), self._turn(k, positions, table, rot_dims)
+            q, k = self._turn(q, positions, table, rot_dims, interleaved), self._turn(k, positions, table, rot_dims, interleaved)
         q_out.copy_(q.reshape(n, q_size).to(q_out.dtype))
         if slot_map is not None:
             page_size = k_pages.shape[2]
@@ -451,7 +480,7 @@ class TorchKernels(KernelSet):
             v_pages[slots // page_size, :, :, slots % page_size] = v.to(v_pages.dtype)
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
-                        chunk, window, sink, out, out_at=0, out_scale=1.0, sink_logits=None, maps=1):
+                        chunk, window, sink, out, out_at=0, out_scale=1.0, sink_logits=None, maps=1, keep_first=0):
         """`maps` > 1: a head has `maps` query vectors; vector number m of a head reads the m-th `dim` columns of its key
         head's record and the head's values.  `sink_logits`: the sink's term is exp(sink_logits[head])."""
         page_size = k_pages.shape[2]
@@ -470,6 +499,8 @@ class TorchKernels(KernelSet):
             if chunk is not None:
                 lowest = max(lowest, history // chunk * chunk)
             key_pos = torch.arange(lowest, length)
+            if keep_first and lowest > 0:       # the request's first keys stay visible behind the window
+                key_pos = torch.cat((torch.arange(0, min(keep_first, lowest)), key_pos))
             pages = table[r][key_pos // page_size].long()
             assert (pages >= 0).all(), "attention would read a page that was given back"
             keys = k_pages[pages, :, key_pos % page_size].float()        # [S, kv_heads, dim]
@@ -478,7 +509,7 @@ class TorchKernels(KernelSet):
             q_pos = history + torch.arange(last - first)
             visible = key_pos[None, :] <= q_pos[:, None]
             if window is not None:
-                visible &= key_pos[None, :] > q_pos[:, None] - window
+                visible &= (key_pos[None, :] > q_pos[:, None] - window) | (key_pos[None, :] < keep_first)
             if chunk is not None:
                 visible &= (key_pos[None, :] // chunk) == (q_pos[:, None] // chunk)
             merged = torch.empty(last - first, q_heads, vdim)
@@ -500,12 +531,14 @@ class TorchKernels(KernelSet):
             out[first:last, out_at:out_at + q_heads * vdim] = (merged.reshape(last - first, q_heads * vdim) * out_scale).to(out.dtype)
 
     def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out, at=0, out_at=0,
-                  out_scale=1.0):
+                  out_scale=1.0, input_activation=None, raw=None):
         n = projected.shape[0]
         qk, vs = heads * dim, heads * vdim
         p = projected[:, at:].float()
         q, k = p[:, :qk].reshape(n, heads, dim), p[:, qk:2 * qk].reshape(n, heads, dim)
         v, g = p[:, 2 * qk:2 * qk + vs].reshape(n, heads, vdim), p[:, 2 * qk + vs:2 * qk + 2 * vs]
+        if input_activation == "silu":
+            q, k, v = q * torch.sigmoid(q), k * torch.sigmoid(k), v * torch.sigmoid(v)
         if rot_dims:
             q, k = self._turn(q, ctx.positions, table, rot_dims), self._turn(k, ctx.positions, table, rot_dims)
         k = k * key_scale
@@ -515,6 +548,9 @@ class TorchKernels(KernelSet):
             for t in range(first, last):
                 S = decay.float()[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
                 o = torch.einsum("hdv,hd->hv", S, q[t])
+                if raw is not None:
+                    raw[t] = o.reshape(-1)
+                    continue
                 o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
                 gate = g[t]
                 out[t, out_at:out_at + vs] = (o.reshape(-1) * gate * torch.sigmoid(gate) * out_scale).to(out.dtype)
@@ -541,12 +577,29 @@ class TorchKernels(KernelSet):
                 out[t] = (S * y[t]).to(out.dtype)
             state[slot, :width] = S
 
-    def route_chosen(self, logits, gates, experts, top):
+    def route_chosen(self, logits, gates, experts, top, law="softmax"):
         values, chosen = logits[:, :experts].topk(top, dim=-1)
         gates.zero_()
+        if law == "sigmoid":
+            gates[:, :experts].scatter_(1, chosen, torch.sigmoid(values))
+            gates[:, experts:] = 1.0
+            return
         gates[:, :experts].scatter_(1, chosen, values.softmax(-1))
         if logits.shape[1] > experts:
             gates[:, experts:] = torch.sigmoid(logits[:, experts:])
+
+    def gate_activation(self, up, gates, act, experts, ff, activation, inside):
+        columns = act.shape[1]
+        weight = gates[:, :experts].repeat_interleave(ff, dim=1)
+        if columns > experts * ff:
+            weight = torch.cat((weight, gates[:, experts:experts + 1].expand(-1, columns - experts * ff)), dim=1)
+        f = {"gelu": lambda z: 0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0))),
+             "gelu_tanh": lambda z: 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3))),
+             "silu": lambda z: z * torch.sigmoid(z),
+             "relu_squared": lambda z: torch.relu(z) ** 2}[activation]
+        z = up.float()
+        value = f(weight * z) if inside else weight * f(z)
+        act.copy_(torch.where(weight != 0, value, torch.zeros_like(value)).to(act.dtype))
 
     def gate_silu_mul(self, gate_up, gates, act, experts, ff):
         columns = act.shape[1]
