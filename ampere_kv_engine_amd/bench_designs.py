@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the Keranex design (and, `--workload tukevik` / `lirulix`, of those designs) at sizes that resemble a real model's layers (random weights),
+"""Prefill and decode throughput of the Keranex design (and, `--workload tukevik` / `lirulix` / `mekuvik`, of those designs) at sizes that resemble a real model's layers (random weights),
 beside the dense Qwen3 decoder at equal width, depth, heads and active feed-forward width - the closest model the
 engine has.  `python bench.py --workload keranex [--design-sizes s,m] [--layers L]` prints one JSON line per size:
 
@@ -113,6 +113,39 @@ def tukevik_beside_lirulix(size: dict, layers: int) -> dict:
                 layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer in (pattern[i % 2] for i in range(layers))])
 
 
+# Mekuvik at the same widths: the pattern [attention over a window that keeps the first tokens + dense feed-forward, linear
+# attention + routed, attention over a latent + routed, linear attention + routed], one norm a layer, all layers inside
+# one pass of the loop; a token uses `top` experts and the shared one, as wide together as the dense feed-forward.  Beside it
+# Tukevik at its size of the same name (the closest design the engine has: the same attention kernels, retention on the
+# same recurrence kernels, routed experts with a shared one through the same products) and Qwen3.
+MEKUVIK_SIZES = {
+    "s": dict(width=2048, vocab=32768, heads=16, kv_heads=4, dim=128, vdim=128, rot=64, window=1024, keep=4, l_heads=16, l_dim=128,
+              l_vdim=128, m_heads=16, m_dim=128, m_rot=64, m_vdim=128, kv_rank=512, q_rank=768, experts=16, top=2, ff=1024,
+              shared=1024, dense=3072),
+    "m": dict(width=4096, vocab=65536, heads=32, kv_heads=8, dim=128, vdim=128, rot=64, window=2048, keep=4, l_heads=32, l_dim=128,
+              l_vdim=128, m_heads=32, m_dim=128, m_rot=64, m_vdim=128, kv_rank=512, q_rank=1536, experts=32, top=4, ff=1024,
+              shared=1024, dense=5120),
+}
+
+
+def mekuvik_config(size: dict, layers: int) -> dict:
+    window = dict(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], vdim=size["vdim"], scale=size["dim"] ** -0.5,
+                  rot=dict(dims=size["rot"], base=1e6), mask=dict(size=size["window"], keep_first=size["keep"]))
+    light = dict(heads=size["l_heads"], dim=size["l_dim"], vdim=size["l_vdim"],
+                 decay=[1.0 - 2.0 ** -(3 + h % 8) for h in range(size["l_heads"])])
+    latent = dict(heads=size["m_heads"], dim=size["m_dim"], rot_dim=size["m_rot"], vdim=size["m_vdim"], kv_rank=size["kv_rank"],
+                  q_rank=size["q_rank"], scale=(size["m_dim"] + size["m_rot"]) ** -0.5,
+                  rot=dict(dims=size["m_rot"], base=1e4, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0)))
+    dense = dict(kind="dense", ff=size["dense"])
+    routed = dict(kind="moe", expert=dict(ff=size["ff"]), router=dict(experts=size["experts"], top=size["top"]),
+                  shared=dict(ff=size["shared"]))
+    pattern = [("attention", window, dense), ("lightning", light, routed), ("latent_attention", latent, routed),
+               ("lightning", light, routed)]
+    return dict(architecture="Mekuvik", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6), logit_scale=0.5,
+                layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer, mlp in (pattern[i % 4] for i in range(layers))],
+                loop=dict(start=0, stop=layers, times=1))
+
+
 def qwen3_beside_tukevik(size: dict, layers: int) -> dict:
     return dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers, hidden_size=size["width"],
                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
@@ -179,7 +212,22 @@ def measure(config, batch: int, context: int, steps: int, warmup: int, graphs: b
 
 def design_workload(sizes: str, layers: int | None, batch: int, context: int, steps: int, warmup: int,
                     graphs: bool = True, only: str = "", design: str = "keranex") -> int:
-    from .config import KeranexConfig, LirulixConfig, Qwen3Config, TukevikConfig
+    from .config import KeranexConfig, LirulixConfig, MekuvikConfig, Qwen3Config, TukevikConfig
+    for name in [s for s in sizes.split(",") if s and design == "mekuvik"]:
+        size, beside = MEKUVIK_SIZES[name], TUKEVIK_SIZES[name]
+        count = layers or 8
+        line = {"workload": "mekuvik", "sizes": name, "layers": count, "batch": batch, "context": context,
+                "prefill_tokens": PREFILL_TOKENS, "dtype": "bf16", "data": "synthetic: random-init weights, random token ids",
+                "shape": size}
+        if only in ("", "mekuvik"):
+            line["mekuvik"] = measure(MekuvikConfig.from_dict(mekuvik_config(size, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "tukevik"):
+            line["tukevik_equal_size"] = measure(TukevikConfig.from_dict(tukevik_config(beside, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "qwen3"):
+            line["qwen3_equal_size"] = measure(Qwen3Config.from_dict(qwen3_beside_tukevik(beside, count)), batch, context, steps, warmup, graphs)
+        print(json.dumps(line), flush=True)
+    if design == "mekuvik":
+        return 0
     for name in [s for s in sizes.split(",") if s and design == "lirulix"]:
         size = LIRULIX_SIZES[name]
         count = layers or 8

@@ -29,25 +29,17 @@ __device__ __forceinline__ void wave_sync_lds() {
 // with 2 i + 1.  With `whole` the root mean square is taken over all of the token's query vectors at once (and over all of
 // its key vectors): every wave sums its side's whole projection for itself.  `q_weight` [q vectors x dim] and `k_weight`
 // [k vectors x dim] (float32, either may be null) multiply the normed values, before the rotation.
+// One (token, item): `which` < q_vectors is a query vector, then the key vectors, then the value heads.  `given` > 0: the
+// factor 1 / rms of the item's side, formed by the caller over the whole projection; else the vector norms itself.
 template <typename T>
-__global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restrict__ projected, long stride, long tokens,
-                                                              int q_heads, int kv_heads, int dim, int vdim, float eps,
-                                                              int normed, const int* __restrict__ slot_map,
-                                                              T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
-                                                              long num_pages, T* __restrict__ q_out, int maps,
-                                                              const float* __restrict__ table, int table_positions,
-                                                              int rot_dims, const int* __restrict__ positions,
-                                                              const float* __restrict__ q_weight,
-                                                              const float* __restrict__ k_weight, int whole,
-                                                              int interleaved) {
-  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+__device__ __forceinline__ void unit_norm_item(const T* __restrict__ row, long n, int which, int lane, int q_heads, int kv_heads,
+                                               int dim, int vdim, float eps, int normed, float given,
+                                               const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                               int page_size, long num_pages, T* __restrict__ q_out, int maps,
+                                               const float* __restrict__ table, int table_positions, int rot_dims,
+                                               const int* __restrict__ positions, const float* __restrict__ q_weight,
+                                               const float* __restrict__ k_weight, int interleaved) {
   const int q_vectors = q_heads * maps, k_vectors = kv_heads * maps;
-  const int items = q_vectors + k_vectors + kv_heads;
-  const long item = static_cast<long>(blockIdx.x) * waves + wave;
-  if (item >= tokens * items) return;
-  const long n = item / items;
-  const int which = static_cast<int>(item % items);
-  const T* row = projected + n * stride;
   if (which < q_vectors + k_vectors) {
     const bool is_q = which < q_vectors;
     const T* x = row + static_cast<long>(which) * dim;       // (key vectors follow the query vectors at the same width)
@@ -63,15 +55,15 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
       y = k_pages + (((page * kv_heads + vector / maps) * page_size + slot % page_size) * maps + vector % maps) * dim;
     }
     float scale = 1.f;
-    if (normed) {
-      const T* side = whole ? row + (is_q ? 0L : static_cast<long>(q_vectors) * dim) : x;
-      const int count = whole ? (is_q ? q_vectors : k_vectors) * dim : dim;
+    if (normed && given > 0.f) {
+      scale = given;
+    } else if (normed) {
       float squares = 0.f;
-      for (int i = lane; i < count; i += kWave) {
-        const float v = to_float(side[i]);
+      for (int i = lane; i < dim; i += kWave) {
+        const float v = to_float(x[i]);
         squares += v * v;
       }
-      scale = rsqrtf(wave_sum(squares) / static_cast<float>(count) + eps);
+      scale = rsqrtf(wave_sum(squares) / static_cast<float>(dim) + eps);
     }
     const float* gain = is_q ? q_weight : k_weight;
     if (gain != nullptr) gain += static_cast<long>(is_q ? which : which - q_vectors) * dim;
@@ -106,6 +98,58 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
     T* y = v_pages + (page * kv_heads + h) * vdim * page_size + slot % page_size;
     for (int i = lane; i < vdim; i += kWave) y[static_cast<long>(i) * page_size] = x[i];
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restrict__ projected, long stride, long tokens,
+                                                              int q_heads, int kv_heads, int dim, int vdim, float eps,
+                                                              int normed, const int* __restrict__ slot_map,
+                                                              T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
+                                                              long num_pages, T* __restrict__ q_out, int maps,
+                                                              const float* __restrict__ table, int table_positions,
+                                                              int rot_dims, const int* __restrict__ positions,
+                                                              const float* __restrict__ q_weight,
+                                                              const float* __restrict__ k_weight, int interleaved) {
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int items = (q_heads + kv_heads) * maps + kv_heads;
+  const long item = static_cast<long>(blockIdx.x) * waves + wave;
+  if (item >= tokens * items) return;
+  const long n = item / items;
+  unit_norm_item<T>(projected + n * stride, n, static_cast<int>(item % items), lane, q_heads, kv_heads, dim, vdim, eps, normed,
+                    0.f, slot_map, k_pages, v_pages, page_size, num_pages, q_out, maps, table, table_positions, rot_dims,
+                    positions, q_weight, k_weight, interleaved);
+}
+
+// The same with the root mean square taken over all of a token's query vectors at once, and over all its key vectors: a
+// block is a token, sums both sides' squares once, and its waves then take the token's items in turn.
+template <typename T>
+__global__ __launch_bounds__(256) void unit_norm_write_whole_kernel(const T* __restrict__ projected, long stride, int q_heads,
+                                                                    int kv_heads, int dim, int vdim, float eps,
+                                                                    const int* __restrict__ slot_map, T* __restrict__ k_pages,
+                                                                    T* __restrict__ v_pages, int page_size, long num_pages,
+                                                                    T* __restrict__ q_out, int maps,
+                                                                    const float* __restrict__ table, int table_positions,
+                                                                    int rot_dims, const int* __restrict__ positions,
+                                                                    const float* __restrict__ q_weight,
+                                                                    const float* __restrict__ k_weight, int interleaved) {
+  __shared__ float scratch[16];
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const long n = blockIdx.x;
+  const T* row = projected + n * stride;
+  const int q_count = q_heads * maps * dim, k_count = kv_heads * maps * dim;
+  float q_squares = 0.f, k_squares = 0.f;
+  for (int i = threadIdx.x; i < q_count + k_count; i += blockDim.x) {
+    const float v = to_float(row[i]);
+    if (i < q_count) q_squares += v * v;
+    else k_squares += v * v;
+  }
+  const float q_scale = rsqrtf(block_sum(q_squares, scratch) / static_cast<float>(q_count) + eps);
+  const float k_scale = rsqrtf(block_sum(k_squares, scratch) / static_cast<float>(k_count) + eps);
+  const int q_vectors = q_heads * maps, items = (q_heads + kv_heads) * maps + kv_heads;
+  for (int which = wave; which < items; which += waves)
+    unit_norm_item<T>(row, n, which, lane, q_heads, kv_heads, dim, vdim, eps, 1, which < q_vectors ? q_scale : k_scale, slot_map,
+                      k_pages, v_pages, page_size, num_pages, q_out, maps, table, table_positions, rot_dims, positions, q_weight,
+                      k_weight, interleaved);
 }
 
 constexpr int kMaxValueRegs = 4;  // value widths up to 256: each lane owns dims lane, lane + 64, ...
@@ -587,11 +631,18 @@ int akv_unit_norm_write(const void* projected, long stride, int dtype, long toke
   if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || maps < 1) return -2;
   if (table != nullptr && (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > dim || positions == nullptr)) return -2;
   const long items = tokens * ((q_heads + kv_heads) * maps + kv_heads);
+  if (whole && normed) {
+    AKV_DISPATCH(dtype, T, unit_norm_write_whole_kernel<T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
+                               static_cast<const T*>(projected), stride, q_heads, kv_heads, dim, vdim, eps, slot_map,
+                               static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages, static_cast<T*>(q_out),
+                               maps, table, table_positions, rot_dims, positions, q_weight, k_weight, interleaved));
+    return AKV_LAUNCH_STATUS();
+  }
   AKV_DISPATCH(dtype, T, unit_norm_write_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(
                              static_cast<const T*>(projected), stride, tokens, q_heads, kv_heads, dim, vdim, eps, normed,
                              slot_map, static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages,
                              static_cast<T*>(q_out), maps, table, table_positions, rot_dims, positions, q_weight,
-                             k_weight, whole, interleaved));
+                             k_weight, interleaved));
   return AKV_LAUNCH_STATUS();
 }
 

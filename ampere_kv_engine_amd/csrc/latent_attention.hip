@@ -637,26 +637,37 @@ __global__ __launch_bounds__(256) void latent_attend_shared_kernel(
 }
 
 // The runs' shares of a column added up: each was formed against its own maximum m; against the largest of them
-// every share counts exp2(m - M) times.  One wave per (tile, column); a lane owns dimensions lane, lane + 64, ...
-__global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
-                                                          int segments, int kv_rank) {
+// every share counts exp2(m - M) times.  One block per (tile, column): the runs' factors are formed once, into LDS; a
+// thread then owns dimensions and adds the runs' values in the order of the runs - loads that wait for nothing but
+// each other's sum.
+constexpr int kMergeRuns = 64;
+__global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
+                                                           int segments, int kv_rank) {
+  __shared__ float factors[kMergeRuns];
+  __shared__ float total_of;
   const long column = blockIdx.x;                   // tile * 16 + rho
   const long tile = column / 16, rho = column % 16;
-  const int lane = threadIdx.x;
-  float top = -INFINITY;
-  for (int p = 0; p < segments; ++p) top = fmaxf(top, parts[((tile * segments + p) * 16 + rho) * (kv_rank + 2) + kv_rank]);
-  float total = 0.f;
-  for (int p = 0; p < segments; ++p) {
-    const float* share = parts + ((tile * segments + p) * 16 + rho) * (kv_rank + 2);
-    if (share[kv_rank] != -INFINITY) total += share[kv_rank + 1] * __builtin_amdgcn_exp2f(share[kv_rank] - top);
+  const float* first = parts + ((tile * segments) * 16 + rho) * (kv_rank + 2);
+  const long step = 16L * (kv_rank + 2);            // from a run's share to the next run's
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    const float m = lane < segments ? first[lane * step + kv_rank] : -INFINITY;
+    const float top = wave_max(m);
+    const float factor = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - top);
+    factors[lane] = factor;
+    const float total = wave_sum(lane < segments && m != -INFINITY ? first[lane * step + kv_rank + 1] * factor : 0.f);
+    if (lane == 0) total_of = total;
   }
-  for (int d = lane; d < kv_rank; d += kWave) {
+  __syncthreads();
+  const float inverse = 1.f / total_of;
+  for (int d = threadIdx.x; d < kv_rank; d += blockDim.x) {
     float acc = 0.f;
+#pragma unroll 8
     for (int p = 0; p < segments; ++p) {
-      const float* share = parts + ((tile * segments + p) * 16 + rho) * (kv_rank + 2);
-      if (share[kv_rank] != -INFINITY) acc += share[d] * __builtin_amdgcn_exp2f(share[kv_rank] - top);
+      const float f = factors[p];
+      acc += f != 0.f ? first[p * step + d] * f : 0.f;
     }
-    out[column * kv_rank + d] = from_float<bf16_t>(acc / total);
+    out[column * kv_rank + d] = from_float<bf16_t>(acc * inverse);
   }
 }
 
@@ -694,8 +705,8 @@ int launch_attend_mfma(const void* q_abs, const void* records, const void* laten
       page_size, num_pages, scale * 1.4426950408889634f, window, segment, segments, parts);
   const int status = AKV_LAUNCH_STATUS();
   if (status != 0 || segments == 1) return status;
-  latent_merge_kernel<<<static_cast<unsigned>(tiles * 16), kWave, 0, stream>>>(parts, static_cast<bf16_t*>(out), segments,
-                                                                              VT * 16);
+  if (segments > kMergeRuns) return -2;
+  latent_merge_kernel<<<static_cast<unsigned>(tiles * 16), 256, 0, stream>>>(parts, static_cast<bf16_t*>(out), segments, VT * 16);
   return AKV_LAUNCH_STATUS();
 }
 

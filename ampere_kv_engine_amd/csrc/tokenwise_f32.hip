@@ -274,6 +274,46 @@ __global__ __launch_bounds__(256) void norm_gate_rows_kernel(const TX* __restric
   }
 }
 
+// The same for rows of up to 256 * 4 * GROUPS values whose width, strides and addresses are multiples of four values: a row
+// stays in registers between its one trip to memory and its store, four values a load.
+template <typename TX, typename T, int GROUPS>
+__global__ __launch_bounds__(256) void norm_gate_rows4_kernel(const TX* __restrict__ x, long x_stride, int width, int normed,
+                                                              const float* __restrict__ weight, float eps,
+                                                              const T* __restrict__ gates, long gate_stride, int gate_act,
+                                                              T* __restrict__ out, long out_stride, float out_scale) {
+  __shared__ float scratch[16];
+  const long n = blockIdx.x;
+  float4 kept[GROUPS], gate[GROUPS];
+#pragma unroll
+  for (int j = 0; j < GROUPS; ++j) {      // (a group beyond the row reads the row's last four values and counts for nothing)
+    const int i = min((j * 256 + static_cast<int>(threadIdx.x)) * 4, width - 4);
+    kept[j] = read4<TX>(x + n * x_stride + i);
+    if (gate_act != 0) gate[j] = read4<T>(gates + n * gate_stride + i);
+  }
+  float scale = out_scale;
+  if (normed) {
+    float squares = 0.f;
+#pragma unroll
+    for (int j = 0; j < GROUPS; ++j)
+      if ((j * 256 + static_cast<int>(threadIdx.x)) * 4 < width)
+        squares += kept[j].x * kept[j].x + kept[j].y * kept[j].y + kept[j].z * kept[j].z + kept[j].w * kept[j].w;
+    scale *= rsqrtf(block_sum(squares, scratch) / static_cast<float>(width) + eps);
+  }
+  auto gated = [gate_act](float g) { return gate_act == 1 ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g)); };
+#pragma unroll
+  for (int j = 0; j < GROUPS; ++j) {
+    const int i = (j * 256 + static_cast<int>(threadIdx.x)) * 4;
+    if (i >= width) continue;
+    float4 v = make_float4(kept[j].x * scale, kept[j].y * scale, kept[j].z * scale, kept[j].w * scale);
+    if (weight != nullptr) {
+      const float4 w = read4<float>(weight + i);
+      v = make_float4(v.x * w.x, v.y * w.y, v.z * w.z, v.w * w.w);
+    }
+    if (gate_act != 0) v = make_float4(v.x * gated(gate[j].x), v.y * gated(gate[j].y), v.z * gated(gate[j].z), v.w * gated(gate[j].w));
+    write4<T>(out + n * out_stride + i, v);
+  }
+}
+
 // ---- a gated feed-forward's activation after a stacked product: out = act(gate) * up --------------------------------------
 __device__ __forceinline__ float gelu_tanh_of(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
@@ -385,16 +425,25 @@ int akv_norm_gate_rows(const void* x, int x_dtype, long x_stride, int width, int
   if (tokens <= 0) return 0;
   if (width <= 0 || gate_act < 0 || gate_act > 2 || (gate_act != 0 && gates == nullptr)) return -2;
   if (x_dtype != kF32 && x_dtype != dtype) return -2;
+  const size_t x_size = x_dtype == kF32 ? 4 : 2, size = dtype == kF32 ? 4 : 2;
+  const bool by_four = width % 4 == 0 && width >= 4 && width <= 256 * 4 * 8 && x_stride % 4 == 0 && out_stride % 4 == 0 &&
+                       (gate_act == 0 || gate_stride % 4 == 0) && reinterpret_cast<uintptr_t>(x) % (4 * x_size) == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % (4 * size) == 0 && reinterpret_cast<uintptr_t>(gates) % (4 * size) == 0 &&
+                       (weight == nullptr || reinterpret_cast<uintptr_t>(weight) % 16 == 0);
+  const unsigned grid = static_cast<unsigned>(tokens);
+#define AKV_ROW_ARGS(TX) static_cast<const TX*>(x), x_stride, width, normed, weight, eps, static_cast<const T*>(gates), gate_stride, gate_act, static_cast<T*>(out), out_stride, out_scale
   AKV_DISPATCH(dtype, T, {
-    if (x_dtype == kF32 && dtype != kF32)
-      norm_gate_rows_kernel<float, T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
-          static_cast<const float*>(x), x_stride, width, normed, weight, eps, static_cast<const T*>(gates), gate_stride,
-          gate_act, static_cast<T*>(out), out_stride, out_scale);
-    else
-      norm_gate_rows_kernel<T, T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
-          static_cast<const T*>(x), x_stride, width, normed, weight, eps, static_cast<const T*>(gates), gate_stride, gate_act,
-          static_cast<T*>(out), out_stride, out_scale);
+    if (x_dtype == kF32 && dtype != kF32) {
+      if (by_four && width <= 256 * 4 * 2) norm_gate_rows4_kernel<float, T, 2><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(float));
+      else if (by_four) norm_gate_rows4_kernel<float, T, 8><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(float));
+      else norm_gate_rows_kernel<float, T><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(float));
+    } else {
+      if (by_four && width <= 256 * 4 * 2) norm_gate_rows4_kernel<T, T, 2><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(T));
+      else if (by_four) norm_gate_rows4_kernel<T, T, 8><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(T));
+      else norm_gate_rows_kernel<T, T><<<grid, 256, 0, stream>>>(AKV_ROW_ARGS(T));
+    }
   });
+#undef AKV_ROW_ARGS
   return AKV_LAUNCH_STATUS();
 }
 

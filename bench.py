@@ -31,6 +31,10 @@ Further workloads run through the scheduler and print a line of their own (`--wo
   lirulix          the Lirulix design (attention with a learned sink, differential attention over a window, the gated
                    delta rule, dense gelu-gated feed-forwards) the same way, beside Tukevik and Qwen3 at equal width,
                    depth, heads and feed-forward width
+  mekuvik          the Mekuvik design (one norm a layer for both branches; attention over a window that keeps the first
+                   tokens, linear attention with a decay per head, gated attention over a latent; routed experts weighted
+                   by sigmoid scores, with a shared one) the same way, beside Tukevik and Qwen3 at equal width, depth,
+                   heads and active feed-forward width
   offline-512-32   the reference's offline batch (docs/BENCHMARK.md:9-24 there) at Qwen3-8B layer sizes: B = 1 and
                    B = 4 requests of 512 input tokens, 32 greedy output tokens each, end-of-sequence ignored; one
                    warm-up, five samples from submission to the last token on the host
@@ -179,11 +183,11 @@ def main() -> int:
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
     parser.add_argument("--mixed-only", action="store_true",
                         help="time the step of 120 prompt tokens beside the batch's decoding requests alone (for kernel profiles)")
-    parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b", "offline-512-32", "keranex", "tukevik", "lirulix"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b", "offline-512-32", "keranex", "tukevik", "lirulix", "mekuvik"], default="decode",
                         help="decode: the headline measurement; keranex: the Keranex design beside Qwen3 at equal size; "
                              "the others run a set of requests through the scheduler")
     parser.add_argument("--design-sizes", default="s,m", help="--workload keranex / tukevik: which of its sizes (s, m)")
-    parser.add_argument("--design-only", default="", choices=["", "keranex", "tukevik", "lirulix", "qwen3"],
+    parser.add_argument("--design-only", default="", choices=["", "keranex", "tukevik", "lirulix", "mekuvik", "qwen3"],
                         help="--workload keranex / tukevik: one of the two models alone (for kernel profiles)")
     parser.add_argument("--library-above", type=int, default=16,
                         help="bfloat16 products of more rows than this go to the BLAS library; -1: none does")
@@ -195,7 +199,7 @@ def main() -> int:
 
     if args.workload == "offline-512-32":
         return offline_workload(args.layers)
-    if args.workload in ("keranex", "tukevik", "lirulix"):
+    if args.workload in ("keranex", "tukevik", "lirulix", "mekuvik"):
         from ampere_kv_engine_amd.bench_designs import design_workload
         return design_workload(args.design_sizes, args.layers, args.batch, min(args.context, SHORT_CONTEXT), args.steps,
                                args.warmup, graphs=not args.no_graphs, only=args.design_only, design=args.workload)
