@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
 // The same with the root mean square taken over all of a token's query vectors at once, and over all its key vectors: a
 // block is a token, sums both sides' squares once, and its waves then take the token's items in turn.
 template <typename T>
-__global__ __launch_bounds__(256) void unit_norm_write_whole_kernel(const T* __restrict__ projected, long stride, int q_heads,
+__global__ __launch_bounds__(1024) void unit_norm_write_whole_kernel(const T* __restrict__ projected, long stride, int q_heads,
                                                                     int kv_heads, int dim, int vdim, float eps,
                                                                     const int* __restrict__ slot_map, T* __restrict__ k_pages,
                                                                     T* __restrict__ v_pages, int page_size, long num_pages,
@@ -632,7 +632,9 @@ int akv_unit_norm_write(const void* projected, long stride, int dtype, long toke
   if (table != nullptr && (rot_dims < 0 || rot_dims % 2 != 0 || rot_dims > dim || positions == nullptr)) return -2;
   const long items = tokens * ((q_heads + kv_heads) * maps + kv_heads);
   if (whole && normed) {
-    AKV_DISPATCH(dtype, T, unit_norm_write_whole_kernel<T><<<static_cast<unsigned>(tokens), 256, 0, stream>>>(
+    // (few tokens: sixteen waves a token share its items; many: four, and the tokens fill the device)
+    const int threads = tokens <= 256 ? 1024 : 256;
+    AKV_DISPATCH(dtype, T, unit_norm_write_whole_kernel<T><<<static_cast<unsigned>(tokens), threads, 0, stream>>>(
                                static_cast<const T*>(projected), stride, q_heads, kv_heads, dim, vdim, eps, slot_map,
                                static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages, static_cast<T*>(q_out),
                                maps, table, table_positions, rot_dims, positions, q_weight, k_weight, interleaved));
