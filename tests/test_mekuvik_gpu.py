@@ -186,6 +186,40 @@ def test_a_random_configuration_through_the_cuttings(seed, tmp_path):
         M.case_mixed_with_pages_and_slots_used_again(engine, case)
 
 
+LONG = {
+    "attention without a window": dict(type="attention", mlp=None, mixer=M.ATTN(4, 2, 32, 16, 0.5, M.ROT(16, 1e4))),
+    "attention over a long window": dict(type="attention", mlp=None, mixer=M.ATTN(6, 3, 16, 24, 0.6, M.ROT(16, 1e5, M.YARN(4.0, 128, 16.0, 1.0)), 200, 7)),
+    "latent attention": dict(type="latent_attention", mlp=None, mixer=M.LATENT(5, 24, 8, 16, 48, 32, 0.3, 1e4, M.YARN(8.0, 64, 32.0, 1.0))),
+    "linear attention": dict(type="lightning", mlp=None, mixer=M.LIGHT(3, 16, 24, (0.97, 0.995, 0.9995))),
+}
+
+
+@pytest.mark.filterwarnings("ignore:a bfloat16 matrix")
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mechanism", list(LONG))
+def test_long_requests_whose_far_keys_count(mechanism, dtype, tmp_path):
+    """One mixer alone, made sharp, over requests of several hundred tokens in pages of 16: a query's few heavy keys lie
+    anywhere in its history (a state carries hundreds of tokens), so a page, a tile of keys or a chunk of the recurrence
+    that went missing far back moves the logits.  Whole, in portions of 2 to 128 tokens, and with the last 40 tokens one by
+    one - where a window of 200 passes over decoded tokens while its seven kept keys stay."""
+    from ampere_kv_engine_amd.config import EngineConfig
+    from ampere_kv_engine_amd.engine import Engine
+    from conftest import random_ids
+    raw = dict(architecture="Mekuvik", vocab=150, width=64, norm=dict(eps=1e-6), logit_scale=0.3, layers=[LONG[mechanism]])
+    folder = M.make_folder(str(tmp_path), raw, 71 + list(LONG).index(mechanism))
+    requests = {"a": random_ids(150, 530, seed=1), "b": random_ids(150, 263, seed=2)}
+    expected = {name: M.plain_logits(folder, ids) for name, ids in requests.items()}
+    engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=16, num_pages=56, max_seqs=4, max_batched_tokens=640,
+                                                     max_seq_len=640, device=DEVICE))
+    for what, schedule in (("whole", schedules.whole(requests)),
+                           ("portions", schedules.portions(requests, sizes=(2, 3, 37, 64, 5, 128, 2, 16, 90, 2))),
+                           ("last tokens one by one", schedules.last_one_by_one(requests, 40))):
+        got, _ = schedules.run(engine, requests, schedule)
+        for name, want in expected.items():
+            M.assert_close(got[name], want, dtype, f"{mechanism}, {what}, request {name}")
+    assert engine.cache.num_free_pages == [56] * len(engine.cache.groups)
+
+
 # ---- the kernels one by one, against the plain functions ----------------------------------------------------------------
 
 def _pages_for(lengths, page, kv_heads, key_width, vdim, dtype):
